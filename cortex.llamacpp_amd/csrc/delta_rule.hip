@@ -1,0 +1,198 @@
+// delta_rule.hip — the gated delta rule: a matrix memory that, per token, decays, corrects what it holds under the token's key towards the token's value,
+// and is read with the token's query.
+//
+// Per value head a state S [D][VD], f32, one per sequence slot (DeltaArgs in kernels.h):
+//     S <- a S            a: one decay per head, or one per key channel (row d of S times a[d])
+//     u  = beta (v - S^T k)
+//     S <- S + k u^T
+//     o  = S^T q          (the read-out sees the token's own write)
+// k is a unit vector, q a unit vector over sqrt(D); both are the silu of a short causal convolution over time of their projections, like v.
+//
+// delta_prep: everything per (token, channel) in front of the recurrence, one launch - the convolution with its silu (inputs before a segment's first row come
+// from the slot's convolution state, which the launch also moves on), beta = sigmoid, the decays a = exp(-exp(A) softplus(pre + dt)).
+// delta_scan: the columns of S evolve independently given k, q, beta and a, so a workgroup owns 64 columns of one head of one sequence segment: lane = column,
+// the 8 or 16 waves split the D rows (each thread keeps its rows of its column in registers).  Per token ONE exchange across the waves: with G = a S the
+// partial sums of G^T k and G^T q are formed in the same pass; u follows from the first, and o = G^T q + u (k . q) needs no second pass over the updated
+// state.  The inputs of CH tokens are staged in LDS at a time and made unit vectors there.  A segment is a run of consecutive batch rows of one sequence - a
+// prompt, a portion of one, a single decoded token: the same code, started from the slot's state and ending with the state written back, so the result does
+// not depend on how a sequence was cut.
+#include "kernels.h"
+
+namespace mi355 {
+
+namespace {
+
+__device__ __forceinline__ float dl_softplus(float z) { return fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z))); }
+
+constexpr int DELTA_PREP_TOKENS = 32;                           // rows of a segment one workgroup of the prep launch walks
+
+// column index -> what it is: [0, C) a convolution channel; [C, C + H) a head's beta; the rest a decay
+__global__ __launch_bounds__(256) void delta_prep_kernel(DeltaArgs a, int C, int NDEC, int move_state) {
+    const int seg = blockIdx.x, col = blockIdx.y * 256 + threadIdx.x;
+    if (col >= C + a.H + NDEC) return;
+    const int start = a.seg_start[seg], len = a.seg_len[seg], slot = a.seg_slot[seg];
+    const int t_lo = blockIdx.z * DELTA_PREP_TOKENS, t_hi = t_lo + DELTA_PREP_TOKENS < len ? t_lo + DELTA_PREP_TOKENS : len;
+    if (col >= C) {
+        const int e = col - C;
+        if (e < a.H) {
+            for (int t = t_lo; t < t_hi; t++) {
+                const float z = a.p[(size_t)(start + t) * a.ld_p + a.off_beta + e];
+                a.c[(size_t)(start + t) * a.ld_c + col] = 1.0f / (1.0f + expf(-z));
+            }
+        } else {
+            const int i = e - a.H, head = a.per_channel ? i / a.D : i;
+            const float rate = expf(a.A_log[head]), bias = a.dt_bias[i];
+            for (int t = t_lo; t < t_hi; t++) a.c[(size_t)(start + t) * a.ld_c + col] = expf(-rate * dl_softplus(a.a[(size_t)(start + t) * a.ld_a + i] + bias));
+        }
+        return;
+    }
+    const int taps = a.taps, back = taps - 1;
+    float w[DELTA_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < DELTA_MAX_TAPS; j++) w[j] = j < taps ? a.conv_w[(size_t)col * taps + j] : 0.0f;
+    float *state = a.conv_state + (size_t)slot * back * C + col;                               // [back][C] of the slot, this channel
+    // the input `ago` tokens before row t of the segment: a row of the batch, or - before the segment's first row - what the slot remembers
+    const auto input = [&](int t) { return t >= 0 ? a.p[(size_t)(start + t) * a.ld_p + col] : state[(size_t)(back + t) * C]; };
+    for (int t = t_lo; t < t_hi; t++) {
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < DELTA_MAX_TAPS; j++)
+            if (j < taps) s = fmaf(w[j], input(t - (back - j)), s);
+        a.c[(size_t)(start + t) * a.ld_c + col] = s / (1.0f + expf(-s));
+    }
+    if (move_state) {                                           // (this workgroup alone reads the segment's old state: every value is read before the first is written)
+        float keep[DELTA_MAX_TAPS - 1];
+#pragma unroll
+        for (int i = 0; i < DELTA_MAX_TAPS - 1; i++) keep[i] = i < back ? input(len - back + i) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < DELTA_MAX_TAPS - 1; i++)
+            if (i < back) state[(size_t)i * C] = keep[i];
+    }
+}
+
+// the convolution state of segments that several workgroups of the prep launch read: moved on by a launch of its own behind it
+__global__ __launch_bounds__(256) void delta_conv_state_kernel(DeltaArgs a, int C) {
+    const int seg = blockIdx.x, col = blockIdx.y * 256 + threadIdx.x;
+    if (col >= C) return;
+    const int start = a.seg_start[seg], len = a.seg_len[seg], slot = a.seg_slot[seg], back = a.taps - 1;
+    float *state = a.conv_state + (size_t)slot * back * C + col;
+    float keep[DELTA_MAX_TAPS - 1];
+#pragma unroll
+    for (int i = 0; i < DELTA_MAX_TAPS - 1; i++) {
+        const int t = len - back + i;
+        keep[i] = i < back ? (t >= 0 ? a.p[(size_t)(start + t) * a.ld_p + col] : state[(size_t)(back + t) * C]) : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < DELTA_MAX_TAPS - 1; i++)
+        if (i < back) state[(size_t)i * C] = keep[i];
+}
+
+template <int DPER, int NDG, bool PERCH>
+__global__ __launch_bounds__(64 * NDG) void delta_scan_kernel(DeltaArgs a) {
+    constexpr int DP = NDG * DPER, CH = 2048 / DP < 32 ? 2048 / DP : 32, NT = 64 * NDG;
+    __shared__ float sq[CH][DP], sk[CH][DP], sa[PERCH ? CH : 1][PERCH ? DP : 1], sv[CH][64], sb[CH][4], red[2][2][NDG][64];
+    const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, j = tid & 63, dg = tid >> 6;
+    const int col = blockIdx.z * 64 + j, d0 = dg * DPER;
+    const int H = a.H, G = a.G, D = a.D, VD = a.VD, kh = h / (H / G);
+    const int start = a.seg_start[seg], len = a.seg_len[seg], slot = a.seg_slot[seg];
+    const int off_k = G * D, off_v = 2 * G * D, off_b = off_v + H * VD, off_a = off_b + H;
+    float *Sg = a.S + ((size_t)slot * H + h) * (size_t)D * VD;
+    float S[DPER];
+#pragma unroll
+    for (int e = 0; e < DPER; e++) S[e] = d0 + e < D && col < VD ? Sg[(size_t)(d0 + e) * VD + col] : 0.0f;
+    const float qscale = 1.0f / sqrtf((float)D);
+    for (int t0 = 0; t0 < len; t0 += CH) {
+        const int nc = len - t0 < CH ? len - t0 : CH;
+        __syncthreads();                                        // (the previous chunk has been used up)
+        for (int idx = tid; idx < nc * DP; idx += NT) {
+            const int tt = idx / DP, d = idx - tt * DP;
+            const float *row = a.c + (size_t)(start + t0 + tt) * a.ld_c;
+            sq[tt][d] = d < D ? row[kh * D + d] : 0.0f;
+            sk[tt][d] = d < D ? row[off_k + kh * D + d] : 0.0f;
+            if (PERCH) sa[tt][d] = d < D ? row[off_a + h * D + d] : 1.0f;
+        }
+        for (int idx = tid; idx < nc * 64; idx += NT) {
+            const int tt = idx >> 6, c = blockIdx.z * 64 + (idx & 63);
+            sv[tt][idx & 63] = c < VD ? a.c[(size_t)(start + t0 + tt) * a.ld_c + off_v + h * VD + c] : 0.0f;
+        }
+        __syncthreads();
+        // unit vectors: a wave per token of the chunk; k . q of the finished vectors goes along (the read-out needs it)
+        for (int tt = dg; tt < nc; tt += NDG) {
+            float qq = 0.0f, kk = 0.0f, kq = 0.0f;
+            for (int d = j; d < D; d += 64) { const float q = sq[tt][d], k = sk[tt][d]; qq = fmaf(q, q, qq); kk = fmaf(k, k, kk); kq = fmaf(k, q, kq); }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) { qq += __shfl_xor(qq, o, 64); kk += __shfl_xor(kk, o, 64); kq += __shfl_xor(kq, o, 64); }
+            const float iq = qscale / sqrtf(qq + 1e-6f), ik = 1.0f / sqrtf(kk + 1e-6f);
+            for (int d = j; d < D; d += 64) { sq[tt][d] *= iq; sk[tt][d] *= ik; }
+            if (j == 0) {
+                const float *row = a.c + (size_t)(start + t0 + tt) * a.ld_c;
+                sb[tt][0] = row[off_b + h];
+                sb[tt][1] = PERCH ? 1.0f : row[off_a + h];
+                sb[tt][2] = kq * iq * ik;
+            }
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nc; tt++) {
+            const float v = sv[tt][j], beta = sb[tt][0], ah = sb[tt][1], kq = sb[tt][2];
+            float sk_ = 0.0f, sq_ = 0.0f;
+#pragma unroll
+            for (int e = 0; e < DPER; e++) {
+                S[e] *= PERCH ? sa[tt][d0 + e] : ah;
+                sk_ = fmaf(S[e], sk[tt][d0 + e], sk_);
+                sq_ = fmaf(S[e], sq[tt][d0 + e], sq_);
+            }
+            const int pb = tt & 1;                              // (two sets of partial sums: one barrier per token is enough)
+            red[pb][0][dg][j] = sk_;
+            red[pb][1][dg][j] = sq_;
+            __syncthreads();
+            float mk = 0.0f, mq = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NDG; w++) { mk += red[pb][0][w][j]; mq += red[pb][1][w][j]; }
+            const float u = beta * (v - mk);
+#pragma unroll
+            for (int e = 0; e < DPER; e++) S[e] = fmaf(sk[tt][d0 + e], u, S[e]);
+            if (dg == 0 && col < VD) a.o[(size_t)(start + t0 + tt) * a.ld_o + (size_t)h * VD + col] = fmaf(u, kq, mq);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < DPER; e++)
+        if (d0 + e < D && col < VD) Sg[(size_t)(d0 + e) * VD + col] = S[e];
+}
+
+template <bool PERCH>
+hipError_t launch_delta_scan_t(const DeltaArgs &a, hipStream_t st) {
+    const dim3 grid((unsigned)a.n_seg, (unsigned)a.H, (unsigned)((a.VD + 63) / 64));
+    // rows of the state per thread x waves per workgroup: the waves split the rows, the more of them the shorter a token's chain
+    if (a.D <= 16) hipLaunchKernelGGL((delta_scan_kernel<2, 8, PERCH>), grid, dim3(512), 0, st, a);
+    else if (a.D <= 32) hipLaunchKernelGGL((delta_scan_kernel<4, 8, PERCH>), grid, dim3(512), 0, st, a);
+    else if (a.D <= 64) hipLaunchKernelGGL((delta_scan_kernel<8, 8, PERCH>), grid, dim3(512), 0, st, a);
+    else if (a.D <= 128) hipLaunchKernelGGL((delta_scan_kernel<8, 16, PERCH>), grid, dim3(1024), 0, st, a);
+    else if (a.D <= 256) hipLaunchKernelGGL((delta_scan_kernel<16, 16, PERCH>), grid, dim3(1024), 0, st, a);
+    else hipLaunchKernelGGL((delta_scan_kernel<32, 16, PERCH>), grid, dim3(1024), 0, st, a);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool delta_shape_ok(int H, int G, int D, int VD, int taps) {
+    return H >= 1 && G >= 1 && H % G == 0 && D >= 1 && D <= 512 && VD >= 1 && taps >= 1 && taps <= DELTA_MAX_TAPS;
+}
+
+hipError_t launch_delta_prep(const DeltaArgs &a, hipStream_t st) {
+    if (a.n_seg <= 0 || a.max_len <= 0) return hipSuccess;
+    if (!delta_shape_ok(a.H, a.G, a.D, a.VD, a.taps)) return hipErrorInvalidValue;
+    const int C = delta_channels(a), NDEC = a.per_channel ? a.H * a.D : a.H;
+    const unsigned chunks = (unsigned)((a.max_len + DELTA_PREP_TOKENS - 1) / DELTA_PREP_TOKENS);
+    const dim3 grid((unsigned)a.n_seg, (unsigned)((C + a.H + NDEC + 255) / 256), chunks);
+    hipLaunchKernelGGL(delta_prep_kernel, grid, dim3(256), 0, st, a, C, NDEC, chunks == 1 && a.taps > 1 ? 1 : 0);
+    if (chunks > 1 && a.taps > 1) hipLaunchKernelGGL(delta_conv_state_kernel, dim3((unsigned)a.n_seg, (unsigned)((C + 255) / 256)), dim3(256), 0, st, a, C);
+    return hipGetLastError();
+}
+
+hipError_t launch_delta_scan(const DeltaArgs &a, hipStream_t st) {
+    if (a.n_seg <= 0) return hipSuccess;
+    if (!delta_shape_ok(a.H, a.G, a.D, a.VD, a.taps)) return hipErrorInvalidValue;
+    return a.per_channel ? launch_delta_scan_t<true>(a, st) : launch_delta_scan_t<false>(a, st);
+}
+
+}  // namespace mi355

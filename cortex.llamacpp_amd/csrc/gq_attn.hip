@@ -2,13 +2,17 @@
 //
 // A token's cache row is [k_0 .. k_{G-1} | v_0 .. v_{G-1}]: G key heads of dim floats, then G value heads of vdim floats; query head h reads key / value
 // head h / (H / G).  Visibility: same sequence, 0 <= pos_query - pos_cell < window (window 0: every earlier cell).  Plain softmax over the visible cells; an
-// optional per-head sink logit joins the denominator; an optional output gate multiplies head h's result by sigmoid(gate[t][h]).  Everything here is f32:
-// positions, angles, norms, scores, weights, the running sums.
+// optional soft cap squashes every score to cap * tanh(score / cap) first; an optional per-head sink logit joins the denominator; an optional output gate
+// multiplies head h's result by sigmoid(gate[t][h]).  Everything here is f32: positions, angles, norms, scores, weights, the running sums.
 //
-// gq_prep: per token, behind the fused q | k | v projection: an optional RMS norm over the WHOLE query projection (all heads at once) and over the whole key
-// projection, with plain weights; the rotation of the first rot_dims entries of every query and key head in the rotate-half layout (entry i pairs with entry
-// i + rot_dims / 2; the per-pair angle table comes from the host); the score multipliers (one number for the layer, one per head) folded into the query;
-// keys and values stored to the token's cache row.
+// gq_prep: per token, behind the fused q | k | v projection: an optional RMS norm of the queries and of the keys with plain weights - over the WHOLE projection
+// (all heads at once) or over every head by itself with one weight vector shared by the heads; the rotation of the first rot_dims entries of every query and
+// key head in the rotate-half layout (entry i pairs with entry i + rot_dims / 2; the per-pair angle table comes from the host); the score multipliers (one
+// number for the layer, one per head) folded into the query; keys and values stored to the token's cache row.
+//
+// Turned values (optional): every value head is stored turned by its own position over all its entries, in the same half-and-half pairing; the weighted sum
+// of a row is turned back by the row's position - each term then carries the turn by (key position - query position), a relative position signal on the
+// value side.  The turn back happens where a row's result is finished: in the per-row kernel, in the merge of split scans, or in gq_unturn behind the tiled pass.
 #include "kernels.h"
 
 namespace mi355 {
@@ -31,24 +35,38 @@ __device__ float gq_block_sum_256(float v, float *sh) {
 constexpr int GQ_MAX_D = 512;                                   // dim and vdim the attention kernel is instantiated for (8 x 64)
 
 __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
+    extern __shared__ float head_inv[];                         // norm per head: [H + G] inverse root mean squares
     __shared__ float sh[4];
     __shared__ float cs[2][GQ_MAX_D / 2];                       // cos / sin of the token's angle per pair: computed once, read by every head
+    __shared__ float csv[2][GQ_MAX_D / 2];                      // the same for the value heads' pairs
     const int t = blockIdx.x, tid = threadIdx.x;
     const int NQ = a.H * a.dim, NK = a.G * a.dim, NV = a.G * a.vdim, half = a.rot_dims >> 1;
     const float *qr = a.p + (size_t)t * a.ld_p, *kr = qr + NQ, *vr = kr + NK;
     float inv_q = 1.0f, inv_k = 1.0f;
-    if (a.wq_norm) {
+    const bool per_head = a.norm_per_head && a.wq_norm && a.wk_norm;
+    if (per_head) {
+        // a wave per head, queries then keys (q | k lie side by side in the row)
+        for (int hh = tid >> 6; hh < a.H + a.G; hh += 4) {
+            const float *src = qr + (size_t)hh * a.dim;
+            float ss = 0.0f;
+            for (int i = tid & 63; i < a.dim; i += 64) { const float v = src[i]; ss = fmaf(v, v, ss); }
+            ss = gq_wave_sum(ss);
+            if ((tid & 63) == 0) head_inv[hh] = 1.0f / sqrtf(ss / (float)a.dim + a.eps);
+        }
+    } else if (a.wq_norm) {
         float ss = 0.0f;
         for (int i = tid; i < NQ; i += 256) { const float v = qr[i]; ss = fmaf(v, v, ss); }
         inv_q = 1.0f / sqrtf(gq_block_sum_256(ss, sh) / (float)NQ + a.eps);
     }
-    if (a.wk_norm) {
+    if (!per_head && a.wk_norm) {
         float ss = 0.0f;
         for (int i = tid; i < NK; i += 256) { const float v = kr[i]; ss = fmaf(v, v, ss); }
         inv_k = 1.0f / sqrtf(gq_block_sum_256(ss, sh) / (float)NK + a.eps);
     }
     const float p = (float)a.tok_pos[t];
     if (tid < half) { const float ang = p * a.rot_freq[tid]; cs[0][tid] = cosf(ang); cs[1][tid] = sinf(ang); }
+    const int vhalf = a.v_rot_freq ? a.vdim >> 1 : 0;
+    if (tid < vhalf) { const float ang = p * a.v_rot_freq[tid]; csv[0][tid] = cosf(ang); csv[1][tid] = sinf(ang); }
     __syncthreads();
     float *qo = a.q + (size_t)t * a.ld_q;
     float *row = a.cache + (size_t)a.tok_cell[t] * (size_t)(NK + NV);
@@ -58,17 +76,18 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
         const int e = isq ? i : i - NQ, d = e % a.dim, b = e - d;
         const float *src = isq ? qr : kr;
         const float *wn = isq ? a.wq_norm : a.wk_norm;
-        const float inv = isq ? inv_q : inv_k;
+        const float inv = per_head ? head_inv[i / a.dim] : isq ? inv_q : inv_k;
+        const int wb = per_head ? 0 : b;                         // (a shared weight vector starts over with every head)
         float o;
         if (d < a.rot_dims) {
             const int j = d < half ? d : d - half;
             const float c = cs[0][j], s = cs[1][j];
             float u = src[b + j] * inv, w = src[b + j + half] * inv;
-            if (wn) { u *= wn[b + j]; w *= wn[b + j + half]; }
+            if (wn) { u *= wn[wb + j]; w *= wn[wb + j + half]; }
             o = d < half ? u * c - w * s : w * c + u * s;
         } else {
             o = src[e] * inv;
-            if (wn) o *= wn[e];
+            if (wn) o *= wn[wb + d];
         }
         if (isq) {
             float m = a.q_scale;
@@ -76,7 +95,35 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
             qo[e] = o * m;
         } else row[e] = o;
     }
-    for (int i = tid; i < NV; i += 256) row[NK + i] = vr[i];
+    if (!a.v_rot_freq) {
+        for (int i = tid; i < NV; i += 256) row[NK + i] = vr[i];
+        return;
+    }
+    for (int i = tid; i < NV; i += 256) {
+        const int d = i % a.vdim, b = i - d;
+        const int j = d < vhalf ? d : d - vhalf;                 // (vdim is even: every entry has a partner)
+        const float c = csv[0][j], s = csv[1][j], u = vr[b + j], w = vr[b + j + vhalf];
+        row[NK + i] = d < vhalf ? u * c - w * s : w * c + u * s;
+    }
+}
+
+// entry i (and its partner i + vdim / 2) of a finished head output: the pair turns back by the row's position
+__device__ __forceinline__ void gq_unturn_pair(float &u, float &w, float pos, float freq) {
+    const float ang = pos * freq, c = cosf(ang), s = sinf(ang);
+    const float x = u * c + w * s, y = w * c - u * s;
+    u = x; w = y;
+}
+
+// behind the tiled pass: out[t][h] turned back in place (the gate, one factor per head, commutes with the turn)
+__global__ __launch_bounds__(256) void gq_unturn_kernel(GqAttnArgs a) {
+    const int t = blockIdx.x, h = blockIdx.y, vhalf = a.vdim >> 1;
+    float *o = a.out + (size_t)t * a.ld_out + (size_t)h * a.vdim;
+    const float pos = (float)a.tok_pos[t];
+    for (int i = threadIdx.x; i < vhalf; i += 256) {
+        float u = o[i], w = o[i + vhalf];
+        gq_unturn_pair(u, w, pos, a.v_rot_freq[i]);
+        o[i] = u; o[i + vhalf] = w;
+    }
 }
 
 // One workgroup per (token, head), NW waves.  A wave works on four cells at a time: each 16-lane group owns one cell, its lanes hold elements
@@ -155,6 +202,7 @@ __global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
         }
 #pragma unroll
         for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);
+        if (a.softcap > 0.0f) dot = a.softcap * tanhf(dot / a.softcap);
         if (vis) {
             const float mn = fmaxf(m, dot), alpha = expf(m - mn), p = expf(dot - mn);   // (m = -inf at the group's first cell: alpha = 0)
             l = l * alpha + p;
@@ -208,6 +256,21 @@ __global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
     for (int w = 0; w < NW; w++) den += wl[w] > 0.0f ? wl[w] * expf(wm[w] - MM) : 0.0f;
     float inv = den > 0.0f ? 1.0f / den : 0.0f;
     if (a.gate) inv *= 1.0f / (1.0f + expf(-a.gate[(size_t)t * a.ld_gate + h]));
+    if (a.v_rot_freq) {                                         // (vdim is even)
+        const int vhalf = VD >> 1;
+        for (int i = tid; i < vhalf; i += blockDim.x) {
+            float o = 0.0f, o2 = 0.0f;
+            for (int w = 0; w < NW; w++) {
+                const float f = wl[w] > 0.0f ? expf(wm[w] - MM) : 0.0f;
+                o += wacc[w * LP + i] * f;
+                o2 += wacc[w * LP + i + vhalf] * f;
+            }
+            gq_unturn_pair(o, o2, (float)tpos, a.v_rot_freq[i]);
+            a.out[(size_t)t * a.ld_out + (size_t)h * VD + i] = o * inv;
+            a.out[(size_t)t * a.ld_out + (size_t)h * VD + i + vhalf] = o2 * inv;
+        }
+        return;
+    }
     for (int i = tid; i < VD; i += blockDim.x) {
         float o = 0.0f;
         for (int w = 0; w < NW; w++) o += wl[w] > 0.0f ? wacc[w * LP + i] * expf(wm[w] - MM) : 0.0f;
@@ -224,6 +287,23 @@ __global__ __launch_bounds__(256) void gq_attn_merge_kernel(GqAttnArgs a, int sp
     for (int s = 0; s < splits; s++) { const float *r = rec + (size_t)s * (VD + 2); den += r[1] > 0.0f ? r[1] * expf(r[0] - MM) : 0.0f; }
     float inv = den > 0.0f ? 1.0f / den : 0.0f;
     if (a.gate) inv *= 1.0f / (1.0f + expf(-a.gate[(size_t)t * a.ld_gate + h]));
+    if (a.v_rot_freq) {                                         // (vdim is even)
+        const int vhalf = VD >> 1;
+        const float pos = (float)a.tok_pos[t];
+        for (int i = tid; i < vhalf; i += 256) {
+            float o = 0.0f, o2 = 0.0f;
+            for (int s = 0; s < splits; s++) {
+                const float *r = rec + (size_t)s * (VD + 2);
+                const float f = r[1] > 0.0f ? expf(r[0] - MM) : 0.0f;
+                o += r[2 + i] * f;
+                o2 += r[2 + i + vhalf] * f;
+            }
+            gq_unturn_pair(o, o2, pos, a.v_rot_freq[i]);
+            a.out[(size_t)t * a.ld_out + (size_t)h * VD + i] = o * inv;
+            a.out[(size_t)t * a.ld_out + (size_t)h * VD + i + vhalf] = o2 * inv;
+        }
+        return;
+    }
     for (int i = tid; i < VD; i += 256) {
         float o = 0.0f;
         for (int s = 0; s < splits; s++) { const float *r = rec + (size_t)s * (VD + 2); o += r[1] > 0.0f ? r[2 + i] * expf(r[0] - MM) : 0.0f; }
@@ -352,6 +432,12 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
                     }
             }
         }
+        if (a.softcap > 0.0f) {
+#pragma unroll
+            for (int i = 0; i < RPT; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) s[i][j] = a.softcap * tanhf(s[i][j] / a.softcap);
+        }
         // ---- the running softmax of each row; P to LDS
 #pragma unroll
         for (int i = 0; i < RPT; i++) {
@@ -437,7 +523,7 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
             den = l[i] * sc + expf(a.sink[h] - MM);
         }
         float inv = den > 0.0f ? sc / den : 0.0f;
-        if (a.gate) inv *= 1.0f / (1.0f + expf(-a.gate[(size_t)r * a.ld_gate + h]));
+        if (a.gate) inv *= 1.0f / (1.0f + expf(-a.gate[(size_t)r * a.ld_gate + h]));   // (a factor per head: it commutes with the turn back that may follow)
 #pragma unroll
         for (int vc = 0; vc < NVC; vc++) {
             const int col = vc * 64 + tc * 4;
@@ -452,6 +538,7 @@ static hipError_t launch_gq_attn_tile(const GqAttnArgs &a, hipStream_t st) {
     if ((long long)((a.T + 63) / 64) * a.H >= 512) {
         const dim3 grid((unsigned)((a.T + 63) / 64), (unsigned)a.H);
         hipLaunchKernelGGL((gq_attn_tile_kernel<NVC, 4>), grid, dim3(256), gqt_lds_floats(64) * sizeof(float), st, a);
+        if (a.v_rot_freq) hipLaunchKernelGGL(gq_unturn_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a);
         return hipGetLastError();
     }
     // too few tiles to fill the device: every tile's chain of cell blocks is cut into runs (at least two blocks each where the cells in use allow), as many
@@ -466,6 +553,7 @@ static hipError_t launch_gq_attn_tile(const GqAttnArgs &a, hipStream_t st) {
     const dim3 grid((unsigned)((a.T + 31) / 32), (unsigned)a.H, (unsigned)splits);
     hipLaunchKernelGGL((gq_attn_tile_kernel<NVC, 2>), grid, dim3(256), gqt_lds_floats(32) * sizeof(float), st, a);
     if (splits > 1) hipLaunchKernelGGL(gq_attn_merge_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a, (int)splits);
+    else if (a.v_rot_freq) hipLaunchKernelGGL(gq_unturn_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a);
     return hipGetLastError();
 }
 
@@ -476,13 +564,15 @@ bool gq_attn_shape_ok(int H, int G, int dim, int vdim) { return H >= 1 && G >= 1
 hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
     if (a.rot_dims < 0 || a.rot_dims > a.dim || a.rot_dims > GQ_MAX_D || (a.rot_dims & 1) || (a.rot_dims > 0 && !a.rot_freq)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(gq_prep_kernel, dim3((unsigned)a.T), dim3(256), 0, st, a);
+    if (a.v_rot_freq && ((a.vdim & 1) || a.vdim > GQ_MAX_D)) return hipErrorInvalidValue;
+    if (a.norm_per_head && (size_t)(a.H + a.G) * sizeof(float) > 32 * 1024) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(gq_prep_kernel, dim3((unsigned)a.T), dim3(256), a.norm_per_head ? (size_t)(a.H + a.G) * sizeof(float) : 0, st, a);
     return hipGetLastError();
 }
 
 hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
-    if (!gq_attn_shape_ok(a.H, a.G, a.dim, a.vdim)) return hipErrorInvalidValue;
+    if (!gq_attn_shape_ok(a.H, a.G, a.dim, a.vdim) || (a.v_rot_freq && (a.vdim & 1))) return hipErrorInvalidValue;
     // batches: the tiled pass (16-byte loads everywhere: head sizes, strides and bases must allow them); a few rows: one workgroup per (row, head)
     const auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (a.T >= GQ_TILE_MIN_ROWS && (a.dim & 3) == 0 && (a.vdim & 3) == 0 && (a.ld_q & 3) == 0 && (a.ld_out & 3) == 0 && al16(a.q) && al16(a.out) && al16(a.cache)) {

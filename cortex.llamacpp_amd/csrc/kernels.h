@@ -195,7 +195,7 @@ hipError_t launch_pack_q80_blocks(const ActQuant &q, int n, int T, uint8_t *bloc
 // regroup ggml rows into the device row layout (Q6_K, Q8_0); other types are byte copies
 hipError_t launch_repack_rows(int type, const uint8_t *src_ggml, uint8_t *dst_dev, int64_t K, int64_t n_rows, hipStream_t st);
 // dst[i][:] = dequant(table row ids[i]) from device-layout rows
-hipError_t launch_get_rows(int type, const uint8_t *table_dev, int64_t K, const int32_t *ids, int n_ids, float *dst, hipStream_t st);
+hipError_t launch_get_rows(int type, const uint8_t *table_dev, int64_t K, const int32_t *ids, int n_ids, float *dst, hipStream_t st, float scale = 1.0f);   // dst = row * scale
 // scratch: cap_rows * 129 words, zero-filled once: [cap_rows ticket words | cap_rows * 64 part values | cap_rows * 64 part indices]; rows <= cap_rows
 hipError_t launch_argmax_rows(const float *x, int n, int rows, int32_t *out, float *scratch, int cap_rows, hipStream_t st);
 // ---- device-side sampling front end (reference call site common_sampler_sample, src/llama_server_context.cc:1679-1698): the k best
@@ -262,7 +262,7 @@ hipError_t launch_moe_scatter_combine(float *x, const float *y, const float *w, 
 // Outer index z < nz, one of: plain strides (x_zs / w_zs / y_zs elements; per-head products); meta != nullptr: z is an expert, its rows of X and Y are
 // [meta[nz + z], + meta[z]) (launch_moe_group's counts | offsets; T = upper bound of any expert's rows); sel != nullptr: z is a (token, rank) pair - weight set
 // sel[z], row z / sel_div of X, row z of Y.
-enum { MMB_STORE = 0, MMB_RELU2 = 1, MMB_SILU_MUL = 2 };       // y | relu(y)^2 | silu(W x) * (W2 x)
+enum { MMB_STORE = 0, MMB_RELU2 = 1, MMB_SILU_MUL = 2, MMB_GELU_MUL = 3 };   // y | relu(y)^2 | silu(W x) * (W2 x) | gelu_tanh(W x) * (W2 x)
 constexpr int MMB_VEC_ROWS = 16;                               // up to this many rows take the one-wave-per-column kernel
 struct MMBArgs {
     const float *x = nullptr; int ldx = 0;
@@ -299,11 +299,15 @@ struct GqPrepArgs {
     const float *p; int ld_p;              // [T][q: H*dim | k: G*dim | v: G*vdim | ...] projections of the batch
     int T, H, G, dim, vdim;
     const float *wq_norm, *wk_norm; float eps;   // nullable: RMS norm over the whole query / key projection (all heads at once), plain weights [H*dim] / [G*dim]
+    int norm_per_head;                     // 1: the statistic is taken over each head's dim entries instead, and the weights are [dim], shared by the heads
     int rot_dims; const float *rot_freq;   // the first rot_dims entries of every q / k head turn, entry i with entry i + rot_dims / 2; [rot_dims / 2] radians per position
     float q_scale; const float *head_scale;      // the query is multiplied by q_scale * head_scale[h] (nullable): the score's constant factors
     const int32_t *tok_pos, *tok_cell;
     float *q; int ld_q;                    // [T][H*dim]: normed, turned, scaled queries
     float *cache;                          // [n_ctx][G*dim + G*vdim]
+    // nullable: [vdim / 2] radians per position - every value head is stored turned by its own position over all its entries (entry m with entry m + vdim / 2);
+    // the attention's output is then turned back by the query's position (GqAttnArgs::v_rot_freq), so that only position differences remain in the sum
+    const float *v_rot_freq;
 };
 hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st);
 struct GqAttnArgs {
@@ -315,6 +319,8 @@ struct GqAttnArgs {
     int window;                            // cells at distance 0 .. window - 1 are seen; 0 = every earlier cell
     const float *sink;                     // [H] or nullptr: a logit without key or value in the softmax denominator
     const float *gate; int ld_gate;        // nullable: head h's output is multiplied by sigmoid(gate[t * ld_gate + h])
+    float softcap;                         // > 0: a score s becomes softcap * tanh(s / softcap) before the softmax
+    const float *v_rot_freq;               // nullable, [vdim / 2]: the values were stored turned (GqPrepArgs); a head's output turns back by minus its row's position, before the gate
     // the scanned cells cut into runs, one workgroup each, merged afterwards: `splits` runs for steps of a few rows; for prompt batches with too few tiles
     // to fill the device as many as n_kv_hint (the host's count of cells in use, 0: unknown) and the buffer allow.  part: room for part_floats floats,
     // T * H * runs * (vdim + 2) are used
@@ -375,9 +381,38 @@ bool mlstm_shape_ok(int D, int VD);
 hipError_t launch_mlstm_gates(const MlstmArgs &a, int T, hipStream_t st);
 hipError_t launch_mlstm_scan(const MlstmArgs &a, hipStream_t st);
 // y[t][h][j] = o / rms(o over the head) * w[h][j] * sigmoid(p[t][off_g + h * VD + j])
+// w_stride: VD (a weight per head and entry) or 0 (one [VD] weight shared by the heads); gate: sigmoid (MLSTM_GATE_SIGMOID) or silu of the pre-activation
+enum { MLSTM_GATE_SIGMOID = 0, MLSTM_GATE_SILU = 1 };
 hipError_t launch_mlstm_out(const float *o, int ld_o, const float *p, int ld_p, int off_g, const float *w, int T, int H, int VD, float eps, float *y, int ld_y,
-                            hipStream_t st);
+                            hipStream_t st, int w_stride = -1, int gate = MLSTM_GATE_SIGMOID);
 hipError_t launch_mlstm_state_reset(float *S, size_t n_s, float *n, size_t n_n, float *m, size_t n_m, hipStream_t st);   // S = 0, n = 0, m = 0
+
+// ---------------------------------------------------------------- gated delta rule (delta_rule.hip)
+// Per head a state matrix S [D][VD], f32, one per sequence slot.  For a token with unit-length key k, unit-length query q / sqrt(D), value v, write strength
+// beta and decay a (one number per head, or one per key channel = row of S):   S <- a S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
+// q, k, v reach the recurrence through a short causal convolution per channel (taps weights, the last one is the current token's) and silu; the last
+// taps - 1 inputs of every channel are part of a slot's state.  H value heads over G query / key heads (head h reads q / k head h / (H / G)).
+constexpr int DELTA_MAX_TAPS = 8;
+struct DeltaArgs {
+    const float *p; int ld_p;              // [T][q: G*D | k: G*D | v: H*VD | ...] projections of the batch, before the convolution
+    int off_beta;                          // column of p with the H write-strength pre-activations
+    const float *a; int ld_a;              // decay pre-activations: [T][H] (per_channel 0) or [T][H*D]
+    int per_channel;
+    const float *A_log, *dt_bias;          // [H]; [H] or [H*D]:  a = exp(-exp(A_log[head]) * softplus(pre + dt_bias))
+    const float *conv_w; int taps;         // [2*G*D + H*VD][taps] f32 (rows in p's channel order)
+    float *conv_state;                     // [slot][taps - 1][2*G*D + H*VD]: the inputs of the last taps - 1 tokens, oldest first
+    float *c; int ld_c;                    // work rows [T][conv + silu of q | k | v ; beta: H ; decay: H or H*D]  (launch_delta_prep writes, the scan reads)
+    float *S;                              // [slot][H][D][VD]
+    float *o; int ld_o;                    // [T][H][VD]
+    int H, G, D, VD;
+    const int32_t *seg_start, *seg_len, *seg_slot; int n_seg;   // runs of consecutive batch rows of one sequence each; no slot twice in a launch
+    int max_len;                           // the longest of these runs (host-side copy of the list)
+};
+inline int delta_channels(const DeltaArgs &a) { return 2 * a.G * a.D + a.H * a.VD; }
+inline int delta_work_row(int H, int G, int D, int VD, int per_channel) { return 2 * G * D + H * VD + H + (per_channel ? H * D : H); }
+bool delta_shape_ok(int H, int G, int D, int VD, int taps);
+hipError_t launch_delta_prep(const DeltaArgs &a, hipStream_t st);    // convolution + silu, beta, decays for the segments' rows; moves the convolution state on
+hipError_t launch_delta_scan(const DeltaArgs &a, hipStream_t st);    // unit q / k and the recurrence, from each slot's state and back into it
 
 // ---------------------------------------------------------------- attention side (attn.hip)
 // words between two merge-ticket counters / hand-over flags of the decode attention kernels (attn_decode_dev.h, attn_out.hip): one 128-byte line each

@@ -108,17 +108,17 @@ hipError_t launch_repack_rows(int type, const uint8_t *src, uint8_t *dst, int64_
 }
 
 // (dequant_elem: one element of a device row - quant_dev.h, shared with the step set-up kernel of attn.hip)
-__global__ void get_rows_kernel(int type, const uint8_t *table, int K, size_t row_bytes, const int32_t *ids, float *dst) {
+__global__ void get_rows_kernel(int type, const uint8_t *table, int K, size_t row_bytes, const int32_t *ids, float *dst, float scale) {
     const int i = blockIdx.y;
     const uint8_t *row = table + (size_t)ids[i] * row_bytes;
     for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < K; e += gridDim.x * blockDim.x)
-        dst[(size_t)i * K + e] = dequant_elem(type, row, K, e);
+        dst[(size_t)i * K + e] = dequant_elem(type, row, K, e) * scale;
 }
-hipError_t launch_get_rows(int type, const uint8_t *table, int64_t K, const int32_t *ids, int n_ids, float *dst, hipStream_t st) {
+hipError_t launch_get_rows(int type, const uint8_t *table, int64_t K, const int32_t *ids, int n_ids, float *dst, hipStream_t st, float scale) {
     if (n_ids <= 0) return hipSuccess;
     int bx = (int)((K + 255) / 256);
     if (bx > 64) bx = 64;
-    hipLaunchKernelGGL(get_rows_kernel, dim3(bx, n_ids), dim3(256), 0, st, type, table, (int)K, dev_row_bytes(type, K), ids, dst);
+    hipLaunchKernelGGL(get_rows_kernel, dim3(bx, n_ids), dim3(256), 0, st, type, table, (int)K, dev_row_bytes(type, K), ids, dst, scale);
     return hipGetLastError();
 }
 

@@ -9,7 +9,8 @@
 // one sequence segment: lane = column, the 8 or 16 waves split the dim rows (each thread keeps its rows of its column - and of n - in registers), the per-token
 // partial sums of S^T q and n . q cross the waves through LDS.  A segment is a run of consecutive rows of the batch that belong to one sequence: a prompt,
 // a portion of one, or a single decoded token - the same code, started from the slot's state and ending with the state written back.
-// mlstm_out: per head, the output divided by its root mean square, times the mixer's norm weight, times sigmoid of the output gate's pre-activation.
+// mlstm_out: per head, the output divided by its root mean square, times the mixer's norm weight (per head and entry, or one vector shared by the heads), times
+// sigmoid - or silu - of the output gate's pre-activation.  The delta-rule mixers close with the same launch.
 #include "kernels.h"
 
 namespace mi355 {
@@ -101,7 +102,7 @@ __global__ void mlstm_gates_kernel(float *p, int ld_p, int off_i, int H, int T, 
 }
 
 __global__ __launch_bounds__(64) void mlstm_out_kernel(const float *o, int ld_o, const float *p, int ld_p, int off_g, const float *w, int H, int VD, float eps,
-                                                       float *y, int ld_y) {
+                                                       float *y, int ld_y, int w_stride, int gate) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const float *orow = o + (size_t)t * ld_o + (size_t)h * VD;
     float ss = 0.0f;
@@ -111,7 +112,8 @@ __global__ __launch_bounds__(64) void mlstm_out_kernel(const float *o, int ld_o,
     const float inv = 1.0f / sqrtf(ss / (float)VD + eps);
     for (int i = lane; i < VD; i += 64) {
         const float g = p[(size_t)t * ld_p + off_g + h * VD + i];
-        y[(size_t)t * ld_y + (size_t)h * VD + i] = orow[i] * inv * w[h * VD + i] * (1.0f / (1.0f + expf(-g)));
+        const float sg = 1.0f / (1.0f + expf(-g));
+        y[(size_t)t * ld_y + (size_t)h * VD + i] = orow[i] * inv * w[h * w_stride + i] * (gate == MLSTM_GATE_SILU ? g * sg : sg);
     }
 }
 
@@ -148,9 +150,9 @@ hipError_t launch_mlstm_scan(const MlstmArgs &a, hipStream_t st) {
 }
 
 hipError_t launch_mlstm_out(const float *o, int ld_o, const float *p, int ld_p, int off_g, const float *w, int T, int H, int VD, float eps, float *y, int ld_y,
-                            hipStream_t st) {
+                            hipStream_t st, int w_stride, int gate) {
     if (T <= 0) return hipSuccess;
-    hipLaunchKernelGGL(mlstm_out_kernel, dim3((unsigned)T, (unsigned)H), dim3(64), 0, st, o, ld_o, p, ld_p, off_g, w, H, VD, eps, y, ld_y);
+    hipLaunchKernelGGL(mlstm_out_kernel, dim3((unsigned)T, (unsigned)H), dim3(64), 0, st, o, ld_o, p, ld_p, off_g, w, H, VD, eps, y, ld_y, w_stride < 0 ? VD : w_stride, gate);
     return hipGetLastError();
 }
 

@@ -13,7 +13,7 @@
 //                 read K-contiguous straight into the matrix-core register layout (lane = (row, k-group of 8)).
 //   * mmb_f32   - batches in f32 mode (and every shape the other two refuse): LDS-tiled, v_fma_f32 only - products of an f32 activation and a bf16 weight
 //                 widened exactly, no reduced-precision matrix mode anywhere.
-// Epilogues: store | relu(y)^2 | silu(W x) * (W2 x) (two weight sets, one pass over the activations).
+// Epilogues: store | relu(y)^2 | silu(W x) * (W2 x) | gelu_tanh(W x) * (W2 x) (the gated ones: two weight sets, one pass over the activations).
 #include "kernels.h"
 
 namespace mi355 {
@@ -36,6 +36,7 @@ __device__ __forceinline__ unsigned short f2bf(float f) {                       
 __device__ __forceinline__ float epi_apply(int epi, float a, float b) {
     if (epi == MMB_RELU2) { const float r = a > 0.0f ? a : 0.0f; return r * r; }
     if (epi == MMB_SILU_MUL) return a / (1.0f + expf(-a)) * b;
+    if (epi == MMB_GELU_MUL) return 0.5f * a * (1.0f + tanhf(0.7978845608028654f * (a + 0.044715f * a * a * a))) * b;   // the tanh form of gelu; sqrt(2 / pi)
     return a;
 }
 
@@ -349,8 +350,8 @@ __global__ __launch_bounds__(256) void mmb_mfma_kernel(MMBArgs a) {
 
 hipError_t launch_mmb(const MMBArgs &a, hipStream_t st) {
     if (a.T <= 0 || a.N <= 0 || a.nz <= 0) return hipSuccess;
-    if (a.K <= 0 || !a.x || !a.w || !a.y || (a.epi == MMB_SILU_MUL && !a.w2)) return hipErrorInvalidValue;
-    const bool gated = a.epi == MMB_SILU_MUL;
+    const bool gated = a.epi == MMB_SILU_MUL || a.epi == MMB_GELU_MUL;
+    if (a.K <= 0 || !a.x || !a.w || !a.y || (gated && !a.w2)) return hipErrorInvalidValue;
     const auto al = [](const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) == 0; };
     // 16-byte loads of both operands: every row start and every stride on a 16-byte boundary
     const bool vec = (a.K % 8) == 0 && (a.ldw % 8) == 0 && (a.w_zs % 8) == 0 && (a.ldx % 4) == 0 && (a.x_zs % 4) == 0 && al(a.w, 16) && al(a.x, 16) &&

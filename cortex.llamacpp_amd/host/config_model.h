@@ -1,5 +1,6 @@
 // config_model.h — what the loaders of the folder models (config.json + model.safetensors, bf16 weights) share: reading the configuration, checking every
-// tensor against it on the way to the device, and laying out the order of layer runs with its looped span.  One loader per design (novorax.cc, fidepel.cc);
+// tensor against it on the way to the device, and laying out the order of layer runs with its looped span.  One loader per design (novorax.cc, fidepel.cc,
+// tuterax.cc);
 // config_model_load picks it by the configuration's "architecture".
 #pragma once
 
@@ -67,6 +68,25 @@ struct Bf16Loader {
         for (int i = 0; i < n; i++) h[(size_t)i] = widen(s[i]);
         return (float *)dev(h.data(), h.size() * 4);
     }
+    // rows of a [rows][K] tensor whose row count the configuration does not name (a low-rank projection's inner size): -1 (err set) if absent or not 2-d
+    int rows_of(const std::string &name, int K) {
+        if (!err.empty()) return -1;
+        const SafeTensor *t = st.find(name);
+        if (!t) { err = "tensor '" + name + "' missing"; return -1; }
+        if (t->shape.size() != 2 || t->shape[1] != K || t->shape[0] < 1 || t->shape[0] > (1 << 24)) { err = "tensor '" + name + "' must be [rows][" + std::to_string(K) + "]"; return -1; }
+        return (int)t->shape[0];
+    }
+    // several [rows_i][K] bf16 tensors under each other, widened to f32 (small per-channel tables a kernel reads as floats)
+    float *rows_f32(const std::vector<std::pair<std::string, int>> &parts, int K) {
+        std::vector<float> host;
+        for (const auto &pr : parts) {
+            const SafeTensor *t = need(pr.first, "BF16", {pr.second, K});
+            if (!t) return nullptr;
+            const unsigned short *s = (const unsigned short *)t->data;
+            for (size_t i = 0; i < (size_t)pr.second * K; i++) host.push_back(widen(s[i]));
+        }
+        return (float *)dev(host.data(), host.size() * 4);
+    }
     // a tensor that holds ONE number, as n copies of it: a norm weight shared by all coordinates takes the kernels' per-coordinate form
     float *scalar_as_vec(const std::string &name, int n) {
         const SafeTensor *t = need(name, "BF16", {});
@@ -114,5 +134,6 @@ bool cfg_layer_runs(const Json &loop, int n_layer, std::string &err, int &times_
 // the designs' loaders: cfg is the parsed config.json of `dir`, ld has model.safetensors open and ld.m set
 Model *novorax_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, std::string &err, int &status);
 Model *fidepel_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, std::string &err, int &status);
+Model *tuterax_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, std::string &err, int &status);
 
 }  // namespace mi355

@@ -1,6 +1,7 @@
 // novorax.cc — the folder models (config.json + model.safetensors): the registry that picks a design's loader by "architecture", the Novorax loader, and what
 // every such design shares inside Context - buffers, cache planes and state slots, segment lists and scan bounds, the layer-run loop, the output head
-// (novorax.h describes the designs, runtime.h the context; the Fidepel loader and its block are in fidepel.cc).
+// (novorax.h describes the designs, runtime.h the context; the Fidepel loader and its block are in fidepel.cc, the Tuterax loader and the delta-rule mixer
+// in tuterax.cc).
 //
 // The context's own machinery carries them: the cell table (find / free / sequence masks) addresses the attention layers' cache planes, the micro-batch staging
 // block brings tokens, positions, cells and sequence ids to the device, the sequence id is the slot of the recurrent state, logits / arg-max / top-k leave
@@ -47,6 +48,7 @@ Model *config_model_load(const std::string &dir, int main_gpu, std::string &err,
     static const struct { const char *architecture; Model *(*build)(const Json &, const std::string &, Bf16Loader &, std::string &, int &); } designs[] = {
         {"Novorax", novorax_build},
         {"Fidepel", fidepel_build},
+        {"Tuterax", tuterax_build},
     };
     status = -102;
     std::ifstream cf(dir + "/config.json");
@@ -226,7 +228,7 @@ Model *novorax_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, st
     int times = 0;
     if (!cfg_layer_runs(cfg["loop"], nl, err, times, [&](int il, int pass) {
             NvxRun r; r.layer = il; r.pass = pass;
-            r.plane = M.layers[(size_t)il].type == NVX_LATENT ? M.n_cache_runs++ : M.n_mlstm_runs++;
+            r.plane = M.layers[(size_t)il].type == NVX_LATENT ? M.n_cache_runs++ : M.n_state_runs++;
             M.runs.push_back(r);
         })) return nullptr;
     if (times > 0) {
@@ -250,6 +252,15 @@ Model *novorax_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, st
 }
 
 // ------------------------------------------------------------------------------------------ context
+// floats one sequence slot holds for a recurrent layer run: the state matrices; the second set (mLSTM: normalisers, delta rule: the convolutions' last
+// taps - 1 inputs); the third (mLSTM: running maxima)
+static void nvx_state_sizes(const NvxLayer &L, size_t &s_sz, size_t &n_sz, size_t &m_sz) {
+    s_sz = (size_t)L.heads * L.dim * L.vdim;
+    if (L.type == NVX_MLSTM) { n_sz = (size_t)L.heads * L.dim; m_sz = (size_t)L.heads; }
+    else { n_sz = (size_t)std::max(L.conv_taps - 1, 0) * (size_t)L.delta_channels(); m_sz = 0; }
+}
+static bool nvx_recurrent(const NvxLayer &L) { return L.type == NVX_MLSTM || L.type == NVX_DELTA; }
+
 bool Context::init_novorax(std::string &err) {
     const NovoraxModel &M = *model->nvx;
     const size_t T = cp.n_ubatch, W = (size_t)M.width, NC = cp.n_ctx, NS = cp.n_seq_max;
@@ -271,17 +282,18 @@ bool Context::init_novorax(std::string &err) {
 
     // cache planes and recurrent state
     nvx_cache_.assign((size_t)M.n_cache_runs, nullptr);
-    nvx_S_.assign((size_t)M.n_mlstm_runs, nullptr); nvx_n_ = nvx_S_; nvx_m_ = nvx_S_;
+    nvx_S_.assign((size_t)M.n_state_runs, nullptr); nvx_n_ = nvx_S_; nvx_m_ = nvx_S_;
     for (const NvxRun &r : M.runs) {
         const NvxLayer &L = M.layers[(size_t)r.layer];
-        if (L.type != NVX_MLSTM) {
+        if (!nvx_recurrent(L)) {
             nvx_cache_[(size_t)r.plane] = (float *)dalloc(NC * (size_t)L.cache_row() * 4);
             if (!nvx_cache_[(size_t)r.plane]) { err = "attention cache allocation failed"; return false; }
         } else {
-            const size_t HS = (size_t)L.heads;
-            nvx_S_[(size_t)r.plane] = (float *)dalloc(NS * HS * L.dim * L.vdim * 4);
-            nvx_n_[(size_t)r.plane] = (float *)dalloc(NS * HS * L.dim * 4);
-            nvx_m_[(size_t)r.plane] = (float *)dalloc(NS * HS * 4);
+            size_t s_sz, n_sz, m_sz;
+            nvx_state_sizes(L, s_sz, n_sz, m_sz);
+            nvx_S_[(size_t)r.plane] = (float *)dalloc(NS * s_sz * 4);
+            nvx_n_[(size_t)r.plane] = (float *)dalloc(std::max<size_t>(NS * n_sz, 1) * 4);
+            nvx_m_[(size_t)r.plane] = (float *)dalloc(std::max<size_t>(NS * m_sz, 1) * 4);
             if (!nvx_S_[(size_t)r.plane] || !nvx_n_[(size_t)r.plane] || !nvx_m_[(size_t)r.plane]) { err = "recurrent state allocation failed"; return false; }
         }
     }
@@ -351,8 +363,9 @@ void Context::nvx_state_reset(int seq) {
     const size_t NS = cp.n_seq_max;
     for (const NvxRun &r : M.runs) {
         const NvxLayer &L = M.layers[(size_t)r.layer];
-        if (L.type != NVX_MLSTM) continue;
-        const size_t s_sz = (size_t)L.heads * L.dim * L.vdim, n_sz = (size_t)L.heads * L.dim, m_sz = (size_t)L.heads;
+        if (!nvx_recurrent(L)) continue;
+        size_t s_sz, n_sz, m_sz;
+        nvx_state_sizes(L, s_sz, n_sz, m_sz);
         const size_t first = seq < 0 ? 0 : (size_t)seq, cnt = seq < 0 ? NS : 1;
         if (first >= NS) continue;
         (void)launch_mlstm_state_reset(nvx_S_[(size_t)r.plane] + first * s_sz, cnt * s_sz, nvx_n_[(size_t)r.plane] + first * n_sz, cnt * n_sz,
@@ -368,11 +381,12 @@ void Context::nvx_state_copy(int src, int dst) {
     if (src < 0 || dst < 0 || (size_t)src >= NS || (size_t)dst >= NS || src == dst) return;
     for (const NvxRun &r : M.runs) {
         const NvxLayer &L = M.layers[(size_t)r.layer];
-        if (L.type != NVX_MLSTM) continue;
-        const size_t s_sz = (size_t)L.heads * L.dim * L.vdim, n_sz = (size_t)L.heads * L.dim, m_sz = (size_t)L.heads;
+        if (!nvx_recurrent(L)) continue;
+        size_t s_sz, n_sz, m_sz;
+        nvx_state_sizes(L, s_sz, n_sz, m_sz);
         (void)hipMemcpyAsync(nvx_S_[(size_t)r.plane] + dst * s_sz, nvx_S_[(size_t)r.plane] + src * s_sz, s_sz * 4, hipMemcpyDeviceToDevice, stream_);
-        (void)hipMemcpyAsync(nvx_n_[(size_t)r.plane] + dst * n_sz, nvx_n_[(size_t)r.plane] + src * n_sz, n_sz * 4, hipMemcpyDeviceToDevice, stream_);
-        (void)hipMemcpyAsync(nvx_m_[(size_t)r.plane] + dst * m_sz, nvx_m_[(size_t)r.plane] + src * m_sz, m_sz * 4, hipMemcpyDeviceToDevice, stream_);
+        if (n_sz) (void)hipMemcpyAsync(nvx_n_[(size_t)r.plane] + dst * n_sz, nvx_n_[(size_t)r.plane] + src * n_sz, n_sz * 4, hipMemcpyDeviceToDevice, stream_);
+        if (m_sz) (void)hipMemcpyAsync(nvx_m_[(size_t)r.plane] + dst * m_sz, nvx_m_[(size_t)r.plane] + src * m_sz, m_sz * 4, hipMemcpyDeviceToDevice, stream_);
     }
     nvx_seq_len_[(size_t)dst] = nvx_seq_len_[(size_t)src];
 }
@@ -449,7 +463,8 @@ hipError_t Context::nvx_feed_forward(const NvxLayer &L, int T) {
     const NovoraxModel &M = *model->nvx;
     const int W = M.width;
     if (L.ff_kind == NVX_FF_DENSE) {
-        NVX_TRY(nvx_linear(L.up, x_, W, T, nvx_ff_, L.ff, MMB_RELU2, nullptr, 1.0f, L.norm2));
+        if (L.gate.w) NVX_TRY(nvx_linear(L.gate, x_, W, T, nvx_ff_, L.ff, MMB_GELU_MUL, &L.up, 1.0f, L.norm2));
+        else NVX_TRY(nvx_linear(L.up, x_, W, T, nvx_ff_, L.ff, MMB_RELU2, nullptr, 1.0f, L.norm2));
         NVX_TRY(nvx_linear(L.down_ff, nvx_ff_, L.ff, T, nvx_y_, W));
         return hipSuccess;
     }
@@ -491,7 +506,7 @@ hipError_t Context::run_layers_novorax(int T) {
     const float eps = M.eps;
     cur_T_ = T;
     NVX_TRY(launch_kv_meta_set(d_cell_pos_, d_cell_seq_, d_cell_, d_pos_, d_seqmask_, T, stream_));
-    NVX_TRY(launch_get_rows(T_BF16, (const uint8_t *)M.embed.w, W, d_tok_, T, x_, stream_));
+    NVX_TRY(launch_get_rows(T_BF16, (const uint8_t *)M.embed.w, W, d_tok_, T, x_, stream_, M.embed_scale));
     if (M.loop_in.w) NVX_TRY(hipMemcpy2DAsync(nvx_xcat_ + W, (size_t)2 * W * 4, x_, (size_t)W * 4, (size_t)W * 4, (size_t)T, hipMemcpyDeviceToDevice, stream_));
     prof_mark("embed");
     int ir = 0;
@@ -553,7 +568,13 @@ hipError_t Context::run_layers_novorax(int T) {
             NVX_TRY(launch_mlstm_out(nvx_o_, H * L.vdim, nvx_a_, LD_P, 2 * H * L.dim + H * L.vdim, L.mix_norm, T, H, L.vdim, eps, nvx_att_, H * L.vdim, stream_));
             NVX_TRY(nvx_linear(L.o, nvx_att_, H * L.vdim, T, nvx_y_, W));
             prof_mark("mlstm");
-        } else return hipErrorInvalidValue;                      // (a mixer this block form has no path for: refused at load)
+        } else if (L.type == NVX_GQ) {
+            NVX_TRY(nvx_linear(L.proj, x_, W, T, nvx_a_, L.proj.N, MMB_STORE, nullptr, 1.0f, L.norm1));
+            NVX_TRY(nvx_gq_attention(L, r, T));
+        } else if (L.type == NVX_DELTA) {
+            NVX_TRY(nvx_delta_mixer(L, r, T));
+        } else return hipErrorInvalidValue;
+        // norm on the sublayer's output, added to the stream (norm1 / norm2 in front of a sublayer are nullptr in a design whose sublayers read the stream itself)
         NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm1b, 1.0f, x_, x_, W, W, T, eps, stream_));
         if (L.ff_kind != NVX_FF_NONE) {
             NVX_TRY(nvx_feed_forward(L, T));

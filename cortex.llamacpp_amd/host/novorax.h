@@ -13,6 +13,13 @@
 // multiplier per head, a sliding window, a sigmoid output gate per head) and whose feed-forward is a routed mixture of relu^2 experts (softmax scores, expert
 // groups of which only the best stay open, renormalised and scaled weights) plus an always-on shared expert; a span of layers may run several times with
 // shared weights and nothing between the passes.
+//
+// Tuterax: every sublayer reads the stream itself and is normed on its OUTPUT (x += norm(mixer(x)), x += norm(ff(x)), zero-centred norm weights).  Mixers:
+// grouped-query attention over every earlier token with RMS-normed queries and keys per head (one weight vector shared by the heads), rotate-half rotary positions
+// on part of each head, values stored turned by their position and the weighted sum turned back by the query's, a soft cap on the scores, a per-head softmax
+// sink; or the gated delta rule (short causal convolutions + silu on q / k / v, unit keys and queries, a write strength beta, a decay per head - "delta" - or per
+// head and key channel through a low-rank projection - "channel_delta" -, per-head unit-RMS output with a silu or a low-rank sigmoid gate).  Feed-forward:
+// W_down (gelu_tanh(W_gate x) * (W_up x)), or none.  The embedding rows enter times a constant and the same table is the output head.
 #pragma once
 
 #include <cstdint>
@@ -26,7 +33,7 @@ struct BfMat {                      // bf16 rows on the device
     int N = 0, K = 0;               // rows (outputs), row length (inputs)
 };
 
-enum { NVX_LATENT = 0, NVX_MLSTM = 1, NVX_GQ = 2 };              // token mixers: latent attention, matrix-memory recurrence, grouped-query attention
+enum { NVX_LATENT = 0, NVX_MLSTM = 1, NVX_GQ = 2, NVX_DELTA = 3 };   // token mixers: latent attention, matrix-memory recurrence, grouped-query attention, gated delta rule
 enum { NVX_FF_NONE = 0, NVX_FF_DENSE = 1, NVX_FF_EXPERTS = 2, NVX_FF_ROUTED = 3 };   // dense; experts by a token-id table; experts by a router
 
 struct NvxLayer {
@@ -51,6 +58,21 @@ struct NvxLayer {
     // (proj above); q_norm / k_norm over the whole projection; head_scale = the per-head score multiplier; the gate and router columns start at off_gate / off_router
     int kv_heads = 0, off_gate = -1, off_router = -1;
     float *q_norm = nullptr, *k_norm = nullptr, *head_scale = nullptr;
+    // ... with q_norm / k_norm per head instead ([dim] weights shared by the heads), a soft cap on the scores (0: none), values stored turned by their position
+    // (v_rot_freq: [vdim / 2] radians per position, nullptr: plain values)
+    bool qk_norm_per_head = false;
+    float softcap = 0.0f;
+    float *v_rot_freq = nullptr;
+    // gated delta rule: proj = [q: kv_heads*dim ; k: kv_heads*dim ; v: heads*vdim ; beta: heads ; then a: heads ; g: heads*vdim  (one decay per head, silu gate)
+    //                                                                               or   a1: rank_a ; g1: rank_g  (decay per key channel and sigmoid gate, both
+    // through a second projection a2 [heads*dim][rank_a], g2 [heads*vdim][rank_g])]; conv_w [2*kv_heads*dim + heads*vdim][conv_taps] f32 in proj's channel order
+    bool decay_per_channel = false;
+    int conv_taps = 0, off_beta = -1, off_a = -1, off_g = -1, rank_a = 0, rank_g = 0;
+    float *conv_w = nullptr, *A_log = nullptr, *dt_bias = nullptr;
+    BfMat a2, g2;
+    // dense feed-forward with a gate: down_ff (act(gate x) * (up x)); gate.w == nullptr: the plain form above
+    BfMat gate;
+    int delta_channels() const { return 2 * kv_heads * dim + heads * vdim; }
     // routed experts (e_up [n_expert][ff][width] with relu^2, e_down [n_expert][width][ff]): groups of neighbouring experts, the `group_keep` best stay open;
     // weights s / sum * router_scale; the shared expert s_up / s_down (shared_ff 0: none) runs for every token
     int n_group = 1, group_keep = 1, shared_ff = 0;
@@ -62,7 +84,7 @@ struct NvxLayer {
 struct NvxRun {
     int layer = 0;
     int pass = -1;                  // >= 0: first layer of loop pass `pass` (input projection + step vector come first)
-    int plane = -1;                 // attention mixers: index of this run's cache plane; mlstm: of its state set
+    int plane = -1;                 // attention mixers: index of this run's cache plane; recurrent mixers: of its state set
 };
 
 struct NovoraxModel {
@@ -71,14 +93,14 @@ struct NovoraxModel {
     BfMat embed, head, loop_in;
     float *loop_step = nullptr;     // [times][width]
     float *final_norm = nullptr;
-    float logit_scale = 1.0f, eps = 1e-5f;
-    std::string design;             // "novorax" | "fidepel"
+    float logit_scale = 1.0f, eps = 1e-5f, embed_scale = 1.0f;
+    std::string design;             // "novorax" | "fidepel" | "tuterax"
     // norm weights: the factor is norm_off + w (1: zero-centred weights, 0: plain ones).  parallel_block: one norm per layer, mixer and feed-forward both read
     // it, x += residual_mult * (their sum); otherwise norms on both sides of each sublayer
     float norm_off = 1.0f, residual_mult = 1.0f;
     bool parallel_block = false;
     int width = 0, n_vocab = 0;
-    int n_cache_runs = 0, n_mlstm_runs = 0;
+    int n_cache_runs = 0, n_state_runs = 0;   // attention runs (cache planes) and recurrent runs (state sets per sequence slot)
     int max_window = 0;             // largest window of the windowed attention layers, 0 if one of them sees every earlier cell (scan bounds)
     int max_shared_ff = 0;
     // largest sizes over the layers (activation buffers)

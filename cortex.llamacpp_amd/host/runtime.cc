@@ -743,7 +743,7 @@ bool Context::kv_seq_rm(int seq, int p0, int p1) {
     if (seq >= 64) return false;                                   // (the cell masks are 64 bits wide)
     if (p0 < 0) p0 = 0;
     if (p1 < 0) p1 = 0x7fffffff;
-    if (model->nvx && model->nvx->n_mlstm_runs > 0) {
+    if (model->nvx && model->nvx->n_state_runs > 0) {
         // a recurrent state cannot be cut back to an earlier position: a sequence goes as a whole (its state slot starts over), or not at all
         for (int sq = 0; sq < (int)nvx_seq_len_.size(); sq++) {
             if (seq >= 0 && sq != seq) continue;

@@ -187,6 +187,7 @@ class Context {
     // fidepel.cc: a block whose mixer and feed-forward read one norm; grouped-query attention on the run's cache plane; experts picked by a router
     hipError_t nvx_parallel_block(const NvxLayer &L, const NvxRun &r, int T);
     hipError_t nvx_gq_attention(const NvxLayer &L, const NvxRun &r, int T);
+    hipError_t nvx_delta_mixer(const NvxLayer &L, const NvxRun &r, int T);   // tuterax.cc: projections, convolution, recurrence, gated unit-RMS output, W_o -> nvx_y_
     hipError_t nvx_routed_experts(const NvxLayer &L, const float *h, const float *pn, int T);
     hipError_t nvx_shared_expert(const NvxLayer &L, const float *h, const float *pn, int T);
     float *nvx_sh_ = nullptr, *nvx_ys_ = nullptr, *nvx_rw_ = nullptr;   // shared expert's hidden rows and output; router weights [T][top]
@@ -200,7 +201,7 @@ class Context {
     void nvx_state_reset(int seq);                          // seq < 0: every slot
     void nvx_state_copy(int src, int dst);
     std::vector<float *> nvx_cache_;                        // [attention run] [n_ctx][the layer's cache_row()]
-    std::vector<float *> nvx_S_, nvx_n_, nvx_m_;            // [mlstm run] [n_seq_max][H][D][VD], [..][H][D], [..][H]
+    std::vector<float *> nvx_S_, nvx_n_, nvx_m_;            // [recurrent run] [n_seq_max][H][D][VD]; mlstm: [..][H][D], [..][H]; delta rule: [..][taps - 1][channels] in nvx_n_
     std::vector<uint64_t> nvx_seq_len_;                     // tokens every sequence id has been fed (the recurrent state cannot be cut back)
     float *nvx_x0_ = nullptr, *nvx_xcat_ = nullptr, *nvx_y_ = nullptr, *nvx_a_ = nullptr, *nvx_cq_ = nullptr, *nvx_q_ = nullptr, *nvx_qa_ = nullptr, *nvx_lat_ = nullptr;
     float *nvx_part_ = nullptr;                             // records of attention scans that were cut into runs (single-token steps; short prompt batches)
