@@ -65,7 +65,9 @@ def sink_softmax(s, seen, sink):
     return e / (e.sum(-1, keepdim=True) + torch.exp(sink - m))
 
 
-def attend(x, W, p, mx, eps):
+def attend(x, W, p, mx, eps, without=()):
+    """`without` names parts to leave out or bend - "sink", "value_turn", "softcap", "causal" (a row then also sees the next position) - so that a test can
+    show that its inputs tell the right mechanism from a wrong one."""
     T = x.shape[0]
     H, G, D, VD = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
     rot = mx.get("rot") or {}
@@ -78,15 +80,20 @@ def attend(x, W, p, mx, eps):
     k = rms_unit(k, eps) * W[p + "k.norm"].to(F64)
     q = turn_halves(q, pos, dims, base)
     k = turn_halves(k, pos, dims, base)
-    v = turn_halves(v, pos, VD, base)
-    seen = pos[None, :] <= pos[:, None]
-    sink = W[p + "sink"].to(F64)
+    turn_v = bool(rot) and "value_turn" not in without
+    if turn_v:
+        v = turn_halves(v, pos, VD, base)
+    seen = pos[None, :] <= pos[:, None] + (1 if "causal" in without else 0)
+    sink = W[p + "sink"].to(F64) if "sink" not in without else torch.full((H,), float("-inf"), dtype=F64)
+    cap = 0.0 if "softcap" in without else float(mx.get("softcap") or 0.0)
     heads = []
     for a in range(H):
         b = a // (H // G)
-        s = softcap((q[:, a] @ k[:, b].T) * float(mx["scale"]), float(mx.get("softcap") or 0.0))
+        s = softcap((q[:, a] @ k[:, b].T) * float(mx.get("scale", 1.0)), cap)
         heads.append(sink_softmax(s, seen, sink[a]) @ v[:, b])
-    o = turn_halves(torch.stack(heads, 1), pos, VD, base, sign=-1.0)
+    o = torch.stack(heads, 1)
+    if turn_v:
+        o = turn_halves(o, pos, VD, base, sign=-1.0)
     return o.reshape(T, H * VD) @ W[p + "o"].to(F64).T
 
 
@@ -153,20 +160,20 @@ def feed_forward(x, W, p):
     return (gelu_tanh(x @ W[p + "gate"].to(F64).T) * (x @ W[p + "up"].to(F64).T)) @ W[p + "down"].to(F64).T
 
 
-def mixer(x, W, p, lc, eps):
+def mixer(x, W, p, lc, eps, without=()):
     if lc["type"] == "attention":
-        return attend(x, W, p, lc["mixer"], eps)
+        return attend(x, W, p, lc["mixer"], eps, without)
     return delta_mixer(x, W, p, lc["mixer"], eps, per_channel=lc["type"] == "channel_delta")
 
 
-def forward(cfg, W, tokens, taps=None):
+def forward(cfg, W, tokens, taps=None, without=()):
     """Logits [T, vocab] of one sequence; taps (a list) receives the stream after every layer."""
     eps = float(cfg["norm"]["eps"])
     E = W["embed"].to(F64)
-    x = E[torch.as_tensor(tokens, dtype=torch.long)] * float(cfg["embedding"]["scale"])
+    x = E[torch.as_tensor(tokens, dtype=torch.long)] * float((cfg.get("embedding") or {}).get("scale", 1.0))
     for il, lc in enumerate(cfg["layers"]):
         p = f"l{il}."
-        x = x + post_norm(mixer(x, W, p + "mix.", lc, eps), W[p + "norm1"], eps)
+        x = x + post_norm(mixer(x, W, p + "mix.", lc, eps, without), W[p + "norm1"], eps)
         if lc.get("mlp"):
             x = x + post_norm(feed_forward(x, W, p + "mlp."), W[p + "norm2"], eps)
         if taps is not None:
