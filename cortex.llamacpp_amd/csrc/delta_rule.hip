@@ -10,10 +10,11 @@
 //
 // delta_prep: everything per (token, channel) in front of the recurrence, one launch - the convolution with its silu (inputs before a segment's first row come
 // from the slot's convolution state, which the launch also moves on), beta = sigmoid, the decays a = exp(-exp(A) softplus(pre + dt)).
-// delta_scan: the columns of S evolve independently given k, q, beta and a, so a workgroup owns 64 columns of one head of one sequence segment: lane = column,
-// the 8 or 16 waves split the D rows (each thread keeps its rows of its column in registers).  Per token ONE exchange across the waves: with G = a S the
-// partial sums of G^T k and G^T q are formed in the same pass; u follows from the first, and o = G^T q + u (k . q) needs no second pass over the updated
-// state.  The inputs of CH tokens are staged in LDS at a time and made unit vectors there.  A segment is a run of consecutive batch rows of one sequence - a
+// delta_scan: the columns of S evolve independently given k, q, beta and a, so a workgroup owns 16 columns of one head of one sequence segment (narrow
+// blocks: a head's state spreads over many compute units, which is what a single sequence has to offer): a wave holds 16 columns x 4 row groups, the 4 or 8
+// waves split the D rows further, each thread keeps its rows of its column in registers.  Per token ONE exchange across the waves: with G = a S the
+// partial sums of G^T k and G^T q are formed in the same pass (row groups meet by lane shuffles, waves through LDS); u follows from the first, and
+// o = G^T q + u (k . q) needs no second pass over the updated state.  The inputs of CH tokens are staged in LDS at a time and made unit vectors there.  A segment is a run of consecutive batch rows of one sequence - a
 // prompt, a portion of one, a single decoded token: the same code, started from the slot's state and ending with the state written back, so the result does
 // not depend on how a sequence was cut.
 #include "kernels.h"
@@ -87,12 +88,17 @@ __global__ __launch_bounds__(256) void delta_conv_state_kernel(DeltaArgs a, int 
         if (i < back) state[(size_t)i * C] = keep[i];
 }
 
-template <int DPER, int NDG, bool PERCH>
-__global__ __launch_bounds__(64 * NDG) void delta_scan_kernel(DeltaArgs a) {
-    constexpr int DP = NDG * DPER, CH = 2048 / DP < 32 ? 2048 / DP : 32, NT = 64 * NDG;
-    __shared__ float sq[CH][DP], sk[CH][DP], sa[PERCH ? CH : 1][PERCH ? DP : 1], sv[CH][64], sb[CH][4], red[2][2][NDG][64];
-    const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, j = tid & 63, dg = tid >> 6;
-    const int col = blockIdx.z * 64 + j, d0 = dg * DPER;
+// lane = (column c of DELTA_COLS, row group rg of DELTA_RG); thread (wave, rg) keeps rows [(wave * DELTA_RG + rg) * DPER, + DPER) of its column
+constexpr int DELTA_COLS = 16, DELTA_RG = 64 / DELTA_COLS;
+
+template <int DPER, int NW, bool PERCH>
+__global__ __launch_bounds__(64 * NW) void delta_scan_kernel(DeltaArgs a) {
+    constexpr int DP = NW * DELTA_RG * DPER, CH = 2048 / DP < 32 ? 2048 / DP : 32, NT = 64 * NW, NLD = (CH * DP + NT - 1) / NT, NLV = (CH * DELTA_COLS + NT - 1) / NT;
+    static_assert(CH <= NT, "one beta / decay load per thread and chunk");
+    __shared__ __attribute__((aligned(16))) float sq[CH][DP], sk[CH][DP], sa[PERCH ? CH : 1][PERCH ? DP : 4];
+    __shared__ float sv[CH][DELTA_COLS], sb[CH][4], red[2][2][NW][DELTA_COLS];
+    const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane % DELTA_COLS, rg = lane / DELTA_COLS;
+    const int col = blockIdx.z * DELTA_COLS + c, d0 = (wave * DELTA_RG + rg) * DPER;
     const int H = a.H, G = a.G, D = a.D, VD = a.VD, kh = h / (H / G);
     const int start = a.seg_start[seg], len = a.seg_len[seg], slot = a.seg_slot[seg];
     const int off_k = G * D, off_v = 2 * G * D, off_b = off_v + H * VD, off_a = off_b + H;
@@ -101,57 +107,96 @@ __global__ __launch_bounds__(64 * NDG) void delta_scan_kernel(DeltaArgs a) {
 #pragma unroll
     for (int e = 0; e < DPER; e++) S[e] = d0 + e < D && col < VD ? Sg[(size_t)(d0 + e) * VD + col] : 0.0f;
     const float qscale = 1.0f / sqrtf((float)D);
+    // a chunk's inputs travel memory -> registers -> LDS; the NEXT chunk's loads are issued before this chunk's tokens are walked, so the chain of tokens
+    // never waits for memory
+    float rq[NLD], rk[NLD], ra[PERCH ? NLD : 1], rv[NLV], rb0 = 0.0f, rb1 = 1.0f;
+    const auto request = [&](int t0) {
+        const int nc = len - t0 < CH ? len - t0 : CH;
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            const int idx = tid + i * NT, tt = idx / DP, d = idx - tt * DP;
+            const bool in = tt < nc && d < D;
+            const float *row = a.c + (size_t)(start + t0 + (tt < nc ? tt : 0)) * a.ld_c;
+            rq[i] = in ? row[kh * D + d] : 0.0f;
+            rk[i] = in ? row[off_k + kh * D + d] : 0.0f;
+            if (PERCH) ra[i] = in ? row[off_a + h * D + d] : 1.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < NLV; i++) {
+            const int idx = tid + i * NT, tt = idx / DELTA_COLS, cc = blockIdx.z * DELTA_COLS + idx % DELTA_COLS;
+            rv[i] = tt < nc && cc < VD ? a.c[(size_t)(start + t0 + tt) * a.ld_c + off_v + h * VD + cc] : 0.0f;
+        }
+        if (tid < nc) {
+            const float *row = a.c + (size_t)(start + t0 + tid) * a.ld_c;
+            rb0 = row[off_b + h];
+            rb1 = PERCH ? 1.0f : row[off_a + h];
+        }
+    };
+    request(0);
     for (int t0 = 0; t0 < len; t0 += CH) {
         const int nc = len - t0 < CH ? len - t0 : CH;
         __syncthreads();                                        // (the previous chunk has been used up)
-        for (int idx = tid; idx < nc * DP; idx += NT) {
-            const int tt = idx / DP, d = idx - tt * DP;
-            const float *row = a.c + (size_t)(start + t0 + tt) * a.ld_c;
-            sq[tt][d] = d < D ? row[kh * D + d] : 0.0f;
-            sk[tt][d] = d < D ? row[off_k + kh * D + d] : 0.0f;
-            if (PERCH) sa[tt][d] = d < D ? row[off_a + h * D + d] : 1.0f;
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            const int idx = tid + i * NT, tt = idx / DP, d = idx - tt * DP;
+            if (tt < CH) { sq[tt][d] = rq[i]; sk[tt][d] = rk[i]; if (PERCH) sa[tt][d] = ra[i]; }
         }
-        for (int idx = tid; idx < nc * 64; idx += NT) {
-            const int tt = idx >> 6, c = blockIdx.z * 64 + (idx & 63);
-            sv[tt][idx & 63] = c < VD ? a.c[(size_t)(start + t0 + tt) * a.ld_c + off_v + h * VD + c] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < NLV; i++) {
+            const int idx = tid + i * NT;
+            if (idx < CH * DELTA_COLS) sv[idx / DELTA_COLS][idx % DELTA_COLS] = rv[i];
         }
+        if (tid < CH) { sb[tid][0] = rb0; sb[tid][1] = rb1; }
+        if (t0 + CH < len) request(t0 + CH);
         __syncthreads();
         // unit vectors: a wave per token of the chunk; k . q of the finished vectors goes along (the read-out needs it)
-        for (int tt = dg; tt < nc; tt += NDG) {
+        for (int tt = wave; tt < nc; tt += NW) {
             float qq = 0.0f, kk = 0.0f, kq = 0.0f;
-            for (int d = j; d < D; d += 64) { const float q = sq[tt][d], k = sk[tt][d]; qq = fmaf(q, q, qq); kk = fmaf(k, k, kk); kq = fmaf(k, q, kq); }
+            for (int d = lane; d < D; d += 64) { const float q = sq[tt][d], k = sk[tt][d]; qq = fmaf(q, q, qq); kk = fmaf(k, k, kk); kq = fmaf(k, q, kq); }
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) { qq += __shfl_xor(qq, o, 64); kk += __shfl_xor(kk, o, 64); kq += __shfl_xor(kq, o, 64); }
             const float iq = qscale / sqrtf(qq + 1e-6f), ik = 1.0f / sqrtf(kk + 1e-6f);
-            for (int d = j; d < D; d += 64) { sq[tt][d] *= iq; sk[tt][d] *= ik; }
-            if (j == 0) {
-                const float *row = a.c + (size_t)(start + t0 + tt) * a.ld_c;
-                sb[tt][0] = row[off_b + h];
-                sb[tt][1] = PERCH ? 1.0f : row[off_a + h];
-                sb[tt][2] = kq * iq * ik;
-            }
+            for (int d = lane; d < D; d += 64) { sq[tt][d] *= iq; sk[tt][d] *= ik; }
+            if (lane == 0) sb[tt][2] = kq * iq * ik;
         }
         __syncthreads();
         for (int tt = 0; tt < nc; tt++) {
-            const float v = sv[tt][j], beta = sb[tt][0], ah = sb[tt][1], kq = sb[tt][2];
-            float sk_ = 0.0f, sq_ = 0.0f;
+            const float v = sv[tt][c], beta = sb[tt][0], ah = sb[tt][1], kq = sb[tt][2];
+            float kv[DPER], qv[DPER], av[DPER];
+            if constexpr (DPER % 4 == 0) {
+#pragma unroll
+                for (int e = 0; e < DPER; e += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4 *>(&sk[tt][d0 + e]), q4 = *reinterpret_cast<const float4 *>(&sq[tt][d0 + e]);
+                    kv[e] = k4.x; kv[e + 1] = k4.y; kv[e + 2] = k4.z; kv[e + 3] = k4.w;
+                    qv[e] = q4.x; qv[e + 1] = q4.y; qv[e + 2] = q4.z; qv[e + 3] = q4.w;
+                    if (PERCH) {
+                        const float4 a4 = *reinterpret_cast<const float4 *>(&sa[tt][d0 + e]);
+                        av[e] = a4.x; av[e + 1] = a4.y; av[e + 2] = a4.z; av[e + 3] = a4.w;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < DPER; e++) { kv[e] = sk[tt][d0 + e]; qv[e] = sq[tt][d0 + e]; if (PERCH) av[e] = sa[tt][d0 + e]; }
+            }
+            float pk = 0.0f, pq = 0.0f;
 #pragma unroll
             for (int e = 0; e < DPER; e++) {
-                S[e] *= PERCH ? sa[tt][d0 + e] : ah;
-                sk_ = fmaf(S[e], sk[tt][d0 + e], sk_);
-                sq_ = fmaf(S[e], sq[tt][d0 + e], sq_);
+                S[e] *= PERCH ? av[e] : ah;
+                pk = fmaf(S[e], kv[e], pk);
+                pq = fmaf(S[e], qv[e], pq);
             }
+#pragma unroll
+            for (int o = DELTA_COLS; o < 64; o <<= 1) { pk += __shfl_xor(pk, o, 64); pq += __shfl_xor(pq, o, 64); }   // the wave's row groups
             const int pb = tt & 1;                              // (two sets of partial sums: one barrier per token is enough)
-            red[pb][0][dg][j] = sk_;
-            red[pb][1][dg][j] = sq_;
+            if (rg == 0) { red[pb][0][wave][c] = pk; red[pb][1][wave][c] = pq; }
             __syncthreads();
             float mk = 0.0f, mq = 0.0f;
 #pragma unroll
-            for (int w = 0; w < NDG; w++) { mk += red[pb][0][w][j]; mq += red[pb][1][w][j]; }
+            for (int w = 0; w < NW; w++) { mk += red[pb][0][w][c]; mq += red[pb][1][w][c]; }
             const float u = beta * (v - mk);
 #pragma unroll
-            for (int e = 0; e < DPER; e++) S[e] = fmaf(sk[tt][d0 + e], u, S[e]);
-            if (dg == 0 && col < VD) a.o[(size_t)(start + t0 + tt) * a.ld_o + (size_t)h * VD + col] = fmaf(u, kq, mq);
+            for (int e = 0; e < DPER; e++) S[e] = fmaf(kv[e], u, S[e]);
+            if (tid < DELTA_COLS && col < VD) a.o[(size_t)(start + t0 + tt) * a.ld_o + (size_t)h * VD + col] = fmaf(u, kq, mq);
         }
     }
 #pragma unroll
@@ -161,14 +206,15 @@ __global__ __launch_bounds__(64 * NDG) void delta_scan_kernel(DeltaArgs a) {
 
 template <bool PERCH>
 hipError_t launch_delta_scan_t(const DeltaArgs &a, hipStream_t st) {
-    const dim3 grid((unsigned)a.n_seg, (unsigned)a.H, (unsigned)((a.VD + 63) / 64));
-    // rows of the state per thread x waves per workgroup: the waves split the rows, the more of them the shorter a token's chain
-    if (a.D <= 16) hipLaunchKernelGGL((delta_scan_kernel<2, 8, PERCH>), grid, dim3(512), 0, st, a);
-    else if (a.D <= 32) hipLaunchKernelGGL((delta_scan_kernel<4, 8, PERCH>), grid, dim3(512), 0, st, a);
-    else if (a.D <= 64) hipLaunchKernelGGL((delta_scan_kernel<8, 8, PERCH>), grid, dim3(512), 0, st, a);
-    else if (a.D <= 128) hipLaunchKernelGGL((delta_scan_kernel<8, 16, PERCH>), grid, dim3(1024), 0, st, a);
-    else if (a.D <= 256) hipLaunchKernelGGL((delta_scan_kernel<16, 16, PERCH>), grid, dim3(1024), 0, st, a);
-    else hipLaunchKernelGGL((delta_scan_kernel<32, 16, PERCH>), grid, dim3(1024), 0, st, a);
+    const dim3 grid((unsigned)a.n_seg, (unsigned)a.H, (unsigned)((a.VD + DELTA_COLS - 1) / DELTA_COLS));
+    // rows of the state per thread x waves per workgroup (x 4 row groups per wave): few waves keep the per-token exchange short, narrow column blocks
+    // spread a head's state over many compute units
+    if (a.D <= 16) hipLaunchKernelGGL((delta_scan_kernel<1, 4, PERCH>), grid, dim3(256), 0, st, a);
+    else if (a.D <= 32) hipLaunchKernelGGL((delta_scan_kernel<2, 4, PERCH>), grid, dim3(256), 0, st, a);
+    else if (a.D <= 64) hipLaunchKernelGGL((delta_scan_kernel<4, 4, PERCH>), grid, dim3(256), 0, st, a);
+    else if (a.D <= 128) hipLaunchKernelGGL((delta_scan_kernel<8, 4, PERCH>), grid, dim3(256), 0, st, a);
+    else if (a.D <= 256) hipLaunchKernelGGL((delta_scan_kernel<8, 8, PERCH>), grid, dim3(512), 0, st, a);
+    else hipLaunchKernelGGL((delta_scan_kernel<16, 8, PERCH>), grid, dim3(512), 0, st, a);
     return hipGetLastError();
 }
 

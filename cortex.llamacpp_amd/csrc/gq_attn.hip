@@ -64,9 +64,9 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
         inv_k = 1.0f / sqrtf(gq_block_sum_256(ss, sh) / (float)NK + a.eps);
     }
     const float p = (float)a.tok_pos[t];
-    if (tid < half) { const float ang = p * a.rot_freq[tid]; cs[0][tid] = cosf(ang); cs[1][tid] = sinf(ang); }
+    if (tid < half) sincosf(p * a.rot_freq[tid], &cs[1][tid], &cs[0][tid]);
     const int vhalf = a.v_rot_freq ? a.vdim >> 1 : 0;
-    if (tid < vhalf) { const float ang = p * a.v_rot_freq[tid]; csv[0][tid] = cosf(ang); csv[1][tid] = sinf(ang); }
+    if (tid < vhalf) sincosf(p * a.v_rot_freq[tid], &csv[1][tid], &csv[0][tid]);
     __syncthreads();
     float *qo = a.q + (size_t)t * a.ld_q;
     float *row = a.cache + (size_t)a.tok_cell[t] * (size_t)(NK + NV);
@@ -109,7 +109,8 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
 
 // entry i (and its partner i + vdim / 2) of a finished head output: the pair turns back by the row's position
 __device__ __forceinline__ void gq_unturn_pair(float &u, float &w, float pos, float freq) {
-    const float ang = pos * freq, c = cosf(ang), s = sinf(ang);
+    float c, s;
+    sincosf(pos * freq, &s, &c);
     const float x = u * c + w * s, y = w * c - u * s;
     u = x; w = y;
 }
