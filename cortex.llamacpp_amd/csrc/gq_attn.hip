@@ -45,13 +45,14 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
     float inv_q = 1.0f, inv_k = 1.0f;
     const bool per_head = a.norm_per_head && a.wq_norm && a.wk_norm;
     if (per_head) {
-        // a wave per head, queries then keys (q | k lie side by side in the row)
-        for (int hh = tid >> 6; hh < a.H + a.G; hh += 4) {
+        // sixteen lanes per head, queries then keys (q | k lie side by side in the row): every lane group's loads are on their way at once
+        for (int hh = tid >> 4; hh < a.H + a.G; hh += 16) {
             const float *src = qr + (size_t)hh * a.dim;
             float ss = 0.0f;
-            for (int i = tid & 63; i < a.dim; i += 64) { const float v = src[i]; ss = fmaf(v, v, ss); }
-            ss = gq_wave_sum(ss);
-            if ((tid & 63) == 0) head_inv[hh] = 1.0f / sqrtf(ss / (float)a.dim + a.eps);
+            for (int i = tid & 15; i < a.dim; i += 16) { const float v = src[i]; ss = fmaf(v, v, ss); }
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            if ((tid & 15) == 0) head_inv[hh] = 1.0f / sqrtf(ss / (float)a.dim + a.eps);
         }
     } else if (a.wq_norm) {
         float ss = 0.0f;
@@ -66,7 +67,15 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
     const float p = (float)a.tok_pos[t];
     if (tid < half) sincosf(p * a.rot_freq[tid], &cs[1][tid], &cs[0][tid]);
     const int vhalf = a.v_rot_freq ? a.vdim >> 1 : 0;
-    if (tid < vhalf) sincosf(p * a.v_rot_freq[tid], &csv[1][tid], &csv[0][tid]);
+    if (tid >= 128 && tid - 128 < vhalf) {                       // (the upper waves: beside the key / query table of the lower ones)
+        const int j = tid - 128;
+        sincosf(p * a.v_rot_freq[j], &csv[1][j], &csv[0][j]);
+        if (a.v_cs) { a.v_cs[(size_t)t * a.vdim + j] = csv[0][j]; a.v_cs[(size_t)t * a.vdim + vhalf + j] = csv[1][j]; }
+    }
+    for (int j = 128 + tid; j < vhalf; j += 256) {              // (value heads beyond 256 entries)
+        sincosf(p * a.v_rot_freq[j], &csv[1][j], &csv[0][j]);
+        if (a.v_cs) { a.v_cs[(size_t)t * a.vdim + j] = csv[0][j]; a.v_cs[(size_t)t * a.vdim + vhalf + j] = csv[1][j]; }
+    }
     __syncthreads();
     float *qo = a.q + (size_t)t * a.ld_q;
     float *row = a.cache + (size_t)a.tok_cell[t] * (size_t)(NK + NV);
@@ -108,9 +117,7 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
 }
 
 // entry i (and its partner i + vdim / 2) of a finished head output: the pair turns back by the row's position
-__device__ __forceinline__ void gq_unturn_pair(float &u, float &w, float pos, float freq) {
-    float c, s;
-    sincosf(pos * freq, &s, &c);
+__device__ __forceinline__ void gq_unturn_pair(float &u, float &w, float c, float s) {
     const float x = u * c + w * s, y = w * c - u * s;
     u = x; w = y;
 }
@@ -119,10 +126,10 @@ __device__ __forceinline__ void gq_unturn_pair(float &u, float &w, float pos, fl
 __global__ __launch_bounds__(256) void gq_unturn_kernel(GqAttnArgs a) {
     const int t = blockIdx.x, h = blockIdx.y, vhalf = a.vdim >> 1;
     float *o = a.out + (size_t)t * a.ld_out + (size_t)h * a.vdim;
-    const float pos = (float)a.tok_pos[t];
+    const float *cs = a.v_cs + (size_t)t * a.vdim;
     for (int i = threadIdx.x; i < vhalf; i += 256) {
         float u = o[i], w = o[i + vhalf];
-        gq_unturn_pair(u, w, pos, a.v_rot_freq[i]);
+        gq_unturn_pair(u, w, cs[i], cs[vhalf + i]);
         o[i] = u; o[i + vhalf] = w;
     }
 }
@@ -257,8 +264,9 @@ __global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
     for (int w = 0; w < NW; w++) den += wl[w] > 0.0f ? wl[w] * expf(wm[w] - MM) : 0.0f;
     float inv = den > 0.0f ? 1.0f / den : 0.0f;
     if (a.gate) inv *= 1.0f / (1.0f + expf(-a.gate[(size_t)t * a.ld_gate + h]));
-    if (a.v_rot_freq) {                                         // (vdim is even)
+    if (a.v_cs) {                                               // (vdim is even)
         const int vhalf = VD >> 1;
+        const float *cs = a.v_cs + (size_t)t * VD;
         for (int i = tid; i < vhalf; i += blockDim.x) {
             float o = 0.0f, o2 = 0.0f;
             for (int w = 0; w < NW; w++) {
@@ -266,7 +274,7 @@ __global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
                 o += wacc[w * LP + i] * f;
                 o2 += wacc[w * LP + i + vhalf] * f;
             }
-            gq_unturn_pair(o, o2, (float)tpos, a.v_rot_freq[i]);
+            gq_unturn_pair(o, o2, cs[i], cs[vhalf + i]);
             a.out[(size_t)t * a.ld_out + (size_t)h * VD + i] = o * inv;
             a.out[(size_t)t * a.ld_out + (size_t)h * VD + i + vhalf] = o2 * inv;
         }
@@ -288,9 +296,9 @@ __global__ __launch_bounds__(256) void gq_attn_merge_kernel(GqAttnArgs a, int sp
     for (int s = 0; s < splits; s++) { const float *r = rec + (size_t)s * (VD + 2); den += r[1] > 0.0f ? r[1] * expf(r[0] - MM) : 0.0f; }
     float inv = den > 0.0f ? 1.0f / den : 0.0f;
     if (a.gate) inv *= 1.0f / (1.0f + expf(-a.gate[(size_t)t * a.ld_gate + h]));
-    if (a.v_rot_freq) {                                         // (vdim is even)
+    if (a.v_cs) {                                               // (vdim is even)
         const int vhalf = VD >> 1;
-        const float pos = (float)a.tok_pos[t];
+        const float *cs = a.v_cs + (size_t)t * VD;
         for (int i = tid; i < vhalf; i += 256) {
             float o = 0.0f, o2 = 0.0f;
             for (int s = 0; s < splits; s++) {
@@ -299,7 +307,7 @@ __global__ __launch_bounds__(256) void gq_attn_merge_kernel(GqAttnArgs a, int sp
                 o += r[2 + i] * f;
                 o2 += r[2 + i + vhalf] * f;
             }
-            gq_unturn_pair(o, o2, pos, a.v_rot_freq[i]);
+            gq_unturn_pair(o, o2, cs[i], cs[vhalf + i]);
             a.out[(size_t)t * a.ld_out + (size_t)h * VD + i] = o * inv;
             a.out[(size_t)t * a.ld_out + (size_t)h * VD + i + vhalf] = o2 * inv;
         }
@@ -539,7 +547,7 @@ static hipError_t launch_gq_attn_tile(const GqAttnArgs &a, hipStream_t st) {
     if ((long long)((a.T + 63) / 64) * a.H >= 512) {
         const dim3 grid((unsigned)((a.T + 63) / 64), (unsigned)a.H);
         hipLaunchKernelGGL((gq_attn_tile_kernel<NVC, 4>), grid, dim3(256), gqt_lds_floats(64) * sizeof(float), st, a);
-        if (a.v_rot_freq) hipLaunchKernelGGL(gq_unturn_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a);
+        if (a.v_cs) hipLaunchKernelGGL(gq_unturn_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a);
         return hipGetLastError();
     }
     // too few tiles to fill the device: every tile's chain of cell blocks is cut into runs (at least two blocks each where the cells in use allow), as many
@@ -554,7 +562,7 @@ static hipError_t launch_gq_attn_tile(const GqAttnArgs &a, hipStream_t st) {
     const dim3 grid((unsigned)((a.T + 31) / 32), (unsigned)a.H, (unsigned)splits);
     hipLaunchKernelGGL((gq_attn_tile_kernel<NVC, 2>), grid, dim3(256), gqt_lds_floats(32) * sizeof(float), st, a);
     if (splits > 1) hipLaunchKernelGGL(gq_attn_merge_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a, (int)splits);
-    else if (a.v_rot_freq) hipLaunchKernelGGL(gq_unturn_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a);
+    else if (a.v_cs) hipLaunchKernelGGL(gq_unturn_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a);
     return hipGetLastError();
 }
 
@@ -565,7 +573,7 @@ bool gq_attn_shape_ok(int H, int G, int dim, int vdim) { return H >= 1 && G >= 1
 hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
     if (a.rot_dims < 0 || a.rot_dims > a.dim || a.rot_dims > GQ_MAX_D || (a.rot_dims & 1) || (a.rot_dims > 0 && !a.rot_freq)) return hipErrorInvalidValue;
-    if (a.v_rot_freq && ((a.vdim & 1) || a.vdim > GQ_MAX_D)) return hipErrorInvalidValue;
+    if (a.v_rot_freq && ((a.vdim & 1) || a.vdim > GQ_MAX_D || !a.v_cs)) return hipErrorInvalidValue;
     if (a.norm_per_head && (size_t)(a.H + a.G) * sizeof(float) > 32 * 1024) return hipErrorInvalidValue;
     hipLaunchKernelGGL(gq_prep_kernel, dim3((unsigned)a.T), dim3(256), a.norm_per_head ? (size_t)(a.H + a.G) * sizeof(float) : 0, st, a);
     return hipGetLastError();
@@ -573,7 +581,7 @@ hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st) {
 
 hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
-    if (!gq_attn_shape_ok(a.H, a.G, a.dim, a.vdim) || (a.v_rot_freq && (a.vdim & 1))) return hipErrorInvalidValue;
+    if (!gq_attn_shape_ok(a.H, a.G, a.dim, a.vdim) || (a.v_cs && (a.vdim & 1))) return hipErrorInvalidValue;
     // batches: the tiled pass (16-byte loads everywhere: head sizes, strides and bases must allow them); a few rows: one workgroup per (row, head)
     const auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (a.T >= GQ_TILE_MIN_ROWS && (a.dim & 3) == 0 && (a.vdim & 3) == 0 && (a.ld_q & 3) == 0 && (a.ld_out & 3) == 0 && al16(a.q) && al16(a.out) && al16(a.cache)) {

@@ -306,8 +306,9 @@ struct GqPrepArgs {
     float *q; int ld_q;                    // [T][H*dim]: normed, turned, scaled queries
     float *cache;                          // [n_ctx][G*dim + G*vdim]
     // nullable: [vdim / 2] radians per position - every value head is stored turned by its own position over all its entries (entry m with entry m + vdim / 2);
-    // the attention's output is then turned back by the query's position (GqAttnArgs::v_rot_freq), so that only position differences remain in the sum
-    const float *v_rot_freq;
+    // the attention's output is then turned back by the query's position, so that only position differences remain in the sum.  v_cs: [T][vdim] - the token's
+    // cos (first vdim / 2) and sin per pair, written here for the attention launch (GqAttnArgs::v_cs)
+    const float *v_rot_freq; float *v_cs;
 };
 hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st);
 struct GqAttnArgs {
@@ -320,7 +321,7 @@ struct GqAttnArgs {
     const float *sink;                     // [H] or nullptr: a logit without key or value in the softmax denominator
     const float *gate; int ld_gate;        // nullable: head h's output is multiplied by sigmoid(gate[t * ld_gate + h])
     float softcap;                         // > 0: a score s becomes softcap * tanh(s / softcap) before the softmax
-    const float *v_rot_freq;               // nullable, [vdim / 2]: the values were stored turned (GqPrepArgs); a head's output turns back by minus its row's position, before the gate
+    const float *v_cs;                     // nullable, [T][vdim] from launch_gq_prep: the values were stored turned; a head's output turns back by minus its row's angle per pair, before the gate
     // the scanned cells cut into runs, one workgroup each, merged afterwards: `splits` runs for steps of a few rows; for prompt batches with too few tiles
     // to fill the device as many as n_kv_hint (the host's count of cells in use, 0: unknown) and the buffer allow.  part: room for part_floats floats,
     // T * H * runs * (vdim + 2) are used

@@ -169,7 +169,7 @@ hipError_t Context::nvx_gq_attention(const NvxLayer &L, const NvxRun &r, int T) 
     GqPrepArgs pa{};
     pa.p = nvx_a_; pa.ld_p = LD_P; pa.T = T; pa.H = H; pa.G = G; pa.dim = L.dim; pa.vdim = L.vdim;
     pa.wq_norm = L.q_norm; pa.wk_norm = L.k_norm; pa.eps = M.eps; pa.rot_dims = L.rot_dims; pa.rot_freq = L.rot_freq;
-    pa.norm_per_head = L.qk_norm_per_head ? 1 : 0; pa.v_rot_freq = L.v_rot_freq;
+    pa.norm_per_head = L.qk_norm_per_head ? 1 : 0; pa.v_rot_freq = L.v_rot_freq; pa.v_cs = L.v_rot_freq ? nvx_vcs_ : nullptr;
     pa.q_scale = L.scale; pa.head_scale = L.head_scale; pa.tok_pos = d_pos_; pa.tok_cell = d_cell_;
     pa.q = nvx_q_; pa.ld_q = H * L.dim; pa.cache = cache;
     FDP_TRY(launch_gq_prep(pa, stream_));
@@ -177,7 +177,7 @@ hipError_t Context::nvx_gq_attention(const NvxLayer &L, const NvxRun &r, int T) 
     aa.q = nvx_q_; aa.ld_q = H * L.dim; aa.out = nvx_att_; aa.ld_out = H * L.vdim; aa.T = T; aa.H = H; aa.G = G; aa.dim = L.dim; aa.vdim = L.vdim;
     aa.cache = cache; aa.cell_pos = d_cell_pos_; aa.cell_seq = d_cell_seq_; aa.tok_pos = d_pos_; aa.tok_seq = d_seq_; aa.n_kv_dev = d_nkv_;
     aa.window = L.window; aa.sink = L.sink; aa.gate = L.off_gate >= 0 ? nvx_a_ + L.off_gate : nullptr; aa.ld_gate = LD_P;
-    aa.softcap = L.softcap; aa.v_rot_freq = L.v_rot_freq;
+    aa.softcap = L.softcap; aa.v_cs = L.v_rot_freq ? nvx_vcs_ : nullptr;
     aa.tok_hi = d_seg_ + 3 * (size_t)cp.n_ubatch;
     aa.tok_lo = M.max_window > 0 ? d_seg_ + 4 * (size_t)cp.n_ubatch : nullptr;
     aa.part = nvx_part_; aa.part_floats = nvx_part_floats_; aa.n_kv_hint = n_kv_;

@@ -323,6 +323,11 @@ bool Context::init_novorax(std::string &err) {
             if (L.type == NVX_GQ) nvx_part_floats_ = std::max(nvx_part_floats_, std::min<size_t>(T, 1024) * (size_t)L.heads * 4 * (size_t)(L.vdim + 2));
         nvx_part_ = (float *)dalloc(nvx_part_floats_ * 4);
     }
+    {
+        int vd = 0;
+        for (const NvxLayer &L : M.layers) if (L.v_rot_freq) vd = std::max(vd, L.vdim);
+        if (vd > 0 && !(nvx_vcs_ = (float *)dalloc(T * (size_t)vd * 4))) { err = "value turn table allocation failed"; return false; }
+    }
     if (!x_ || !xn_ || !xo_ || !nvx_x0_ || !nvx_xcat_ || !nvx_y_ || !nvx_a_ || !nvx_cq_ || !nvx_q_ || !nvx_qa_ || !nvx_lat_ || !nvx_att_ || !nvx_o_ || !nvx_ff_) { err = "activation buffer allocation failed"; return false; }
     if (M.max_top > 0) {
         nvx_xg_ = (float *)dalloc(T * TOP * W * 4);

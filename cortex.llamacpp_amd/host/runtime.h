@@ -204,6 +204,7 @@ class Context {
     std::vector<float *> nvx_S_, nvx_n_, nvx_m_;            // [recurrent run] [n_seq_max][H][D][VD]; mlstm: [..][H][D], [..][H]; delta rule: [..][taps - 1][channels] in nvx_n_
     std::vector<uint64_t> nvx_seq_len_;                     // tokens every sequence id has been fed (the recurrent state cannot be cut back)
     float *nvx_x0_ = nullptr, *nvx_xcat_ = nullptr, *nvx_y_ = nullptr, *nvx_a_ = nullptr, *nvx_cq_ = nullptr, *nvx_q_ = nullptr, *nvx_qa_ = nullptr, *nvx_lat_ = nullptr;
+    float *nvx_vcs_ = nullptr;                              // [n_ubatch][widest turned value head]: cos | sin per pair of every token's value turn
     float *nvx_part_ = nullptr;                             // records of attention scans that were cut into runs (single-token steps; short prompt batches)
     size_t nvx_part_floats_ = 0;
     float *nvx_att_ = nullptr, *nvx_o_ = nullptr, *nvx_ff_ = nullptr, *nvx_xg_ = nullptr, *nvx_yg_ = nullptr;
