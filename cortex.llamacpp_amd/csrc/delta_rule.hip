@@ -88,6 +88,18 @@ __global__ __launch_bounds__(256) void delta_conv_state_kernel(DeltaArgs a, int 
         if (i < back) state[(size_t)i * C] = keep[i];
 }
 
+// x summed over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the row groups of a column), the same bits in all four: the lane-swap instructions of gfx950
+// exchange 16-lane (32-lane) rows between two registers - with both operands x the two results are x and its partner, in every lane
+__device__ __forceinline__ float delta_rows_sum(float x) {
+    static_assert(64 / 16 == 4, "four row groups of sixteen columns");
+    const unsigned a = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane16_swap(a, a, false, false);
+    const float y = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    const unsigned b = __float_as_uint(y);
+    const auto q = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+    return __uint_as_float(q[0]) + __uint_as_float(q[1]);
+}
+
 // lane = (column c of DELTA_COLS, row group rg of DELTA_RG); thread (wave, rg) keeps rows [(wave * DELTA_RG + rg) * DPER, + DPER) of its column
 constexpr int DELTA_COLS = 16, DELTA_RG = 64 / DELTA_COLS;
 
@@ -149,46 +161,62 @@ __global__ __launch_bounds__(64 * NW) void delta_scan_kernel(DeltaArgs a) {
         if (tid < CH) { sb[tid][0] = rb0; sb[tid][1] = rb1; }
         if (t0 + CH < len) request(t0 + CH);
         __syncthreads();
-        // unit vectors: a wave per token of the chunk; k . q of the finished vectors goes along (the read-out needs it)
-        for (int tt = wave; tt < nc; tt += NW) {
+        // unit vectors: sixteen lanes per token, four tokens of the chunk per wave at a time; k . q of the finished vectors goes along (the read-out needs it)
+        for (int base = wave * 4; base < nc; base += NW * 4) {
+            const int tt = base + (lane >> 4), li = lane & 15;
+            const bool live = tt < nc;
             float qq = 0.0f, kk = 0.0f, kq = 0.0f;
-            for (int d = lane; d < D; d += 64) { const float q = sq[tt][d], k = sk[tt][d]; qq = fmaf(q, q, qq); kk = fmaf(k, k, kk); kq = fmaf(k, q, kq); }
+            if (live)
+                for (int d = li; d < D; d += 16) { const float q = sq[tt][d], k = sk[tt][d]; qq = fmaf(q, q, qq); kk = fmaf(k, k, kk); kq = fmaf(k, q, kq); }
 #pragma unroll
-            for (int o = 32; o > 0; o >>= 1) { qq += __shfl_xor(qq, o, 64); kk += __shfl_xor(kk, o, 64); kq += __shfl_xor(kq, o, 64); }
+            for (int o = 8; o > 0; o >>= 1) { qq += __shfl_xor(qq, o, 64); kk += __shfl_xor(kk, o, 64); kq += __shfl_xor(kq, o, 64); }
             const float iq = qscale / sqrtf(qq + 1e-6f), ik = 1.0f / sqrtf(kk + 1e-6f);
-            for (int d = lane; d < D; d += 64) { sq[tt][d] *= iq; sk[tt][d] *= ik; }
-            if (lane == 0) sb[tt][2] = kq * iq * ik;
+            if (live) {
+                for (int d = li; d < D; d += 16) { sq[tt][d] *= iq; sk[tt][d] *= ik; }
+                if (li == 0) sb[tt][2] = kq * iq * ik;
+            }
         }
         __syncthreads();
-        for (int tt = 0; tt < nc; tt++) {
-            const float v = sv[tt][c], beta = sb[tt][0], ah = sb[tt][1], kq = sb[tt][2];
-            float kv[DPER], qv[DPER], av[DPER];
+        // the walk: a token's k / q / a / v / beta are in registers BEFORE the barrier of the token in front of it, so that behind the barrier only the
+        // exchanged sums, u and the update stand between one token and the next
+        float kv[DPER], qv[DPER], av[PERCH ? DPER : 1], v, beta, ah, kq;
+        const auto fetch = [&](int tt, float (&k_)[DPER], float (&q_)[DPER], float (&a_)[PERCH ? DPER : 1], float &v_, float &b_, float &ah_, float &kq_) {
+            v_ = sv[tt][c]; b_ = sb[tt][0]; ah_ = sb[tt][1]; kq_ = sb[tt][2];
             if constexpr (DPER % 4 == 0) {
 #pragma unroll
                 for (int e = 0; e < DPER; e += 4) {
                     const float4 k4 = *reinterpret_cast<const float4 *>(&sk[tt][d0 + e]), q4 = *reinterpret_cast<const float4 *>(&sq[tt][d0 + e]);
-                    kv[e] = k4.x; kv[e + 1] = k4.y; kv[e + 2] = k4.z; kv[e + 3] = k4.w;
-                    qv[e] = q4.x; qv[e + 1] = q4.y; qv[e + 2] = q4.z; qv[e + 3] = q4.w;
-                    if (PERCH) {
+                    k_[e] = k4.x; k_[e + 1] = k4.y; k_[e + 2] = k4.z; k_[e + 3] = k4.w;
+                    q_[e] = q4.x; q_[e + 1] = q4.y; q_[e + 2] = q4.z; q_[e + 3] = q4.w;
+                    if constexpr (PERCH) {
                         const float4 a4 = *reinterpret_cast<const float4 *>(&sa[tt][d0 + e]);
-                        av[e] = a4.x; av[e + 1] = a4.y; av[e + 2] = a4.z; av[e + 3] = a4.w;
+                        a_[e] = a4.x; a_[e + 1] = a4.y; a_[e + 2] = a4.z; a_[e + 3] = a4.w;
                     }
                 }
             } else {
 #pragma unroll
-                for (int e = 0; e < DPER; e++) { kv[e] = sk[tt][d0 + e]; qv[e] = sq[tt][d0 + e]; if (PERCH) av[e] = sa[tt][d0 + e]; }
+                for (int e = 0; e < DPER; e++) {
+                    k_[e] = sk[tt][d0 + e]; q_[e] = sq[tt][d0 + e];
+                    if constexpr (PERCH) a_[e] = sa[tt][d0 + e];
+                }
             }
+        };
+        fetch(0, kv, qv, av, v, beta, ah, kq);
+        for (int tt = 0; tt < nc; tt++) {
             float pk = 0.0f, pq = 0.0f;
 #pragma unroll
             for (int e = 0; e < DPER; e++) {
-                S[e] *= PERCH ? av[e] : ah;
+                float decay = ah;
+                if constexpr (PERCH) decay = av[e];
+                S[e] *= decay;
                 pk = fmaf(S[e], kv[e], pk);
                 pq = fmaf(S[e], qv[e], pq);
             }
-#pragma unroll
-            for (int o = DELTA_COLS; o < 64; o <<= 1) { pk += __shfl_xor(pk, o, 64); pq += __shfl_xor(pq, o, 64); }   // the wave's row groups
+            pk = delta_rows_sum(pk); pq = delta_rows_sum(pq);   // the wave's four row groups
             const int pb = tt & 1;                              // (two sets of partial sums: one barrier per token is enough)
             if (rg == 0) { red[pb][0][wave][c] = pk; red[pb][1][wave][c] = pq; }
+            float kn[DPER], qn[DPER], an[PERCH ? DPER : 1], vn = 0.0f, bn = 0.0f, ahn = 1.0f, kqn = 0.0f;
+            if (tt + 1 < nc) fetch(tt + 1, kn, qn, an, vn, bn, ahn, kqn);
             __syncthreads();
             float mk = 0.0f, mq = 0.0f;
 #pragma unroll
@@ -197,6 +225,11 @@ __global__ __launch_bounds__(64 * NW) void delta_scan_kernel(DeltaArgs a) {
 #pragma unroll
             for (int e = 0; e < DPER; e++) S[e] = fmaf(kv[e], u, S[e]);
             if (tid < DELTA_COLS && col < VD) a.o[(size_t)(start + t0 + tt) * a.ld_o + (size_t)h * VD + col] = fmaf(u, kq, mq);
+            if (tt + 1 < nc) {
+#pragma unroll
+                for (int e = 0; e < DPER; e++) { kv[e] = kn[e]; qv[e] = qn[e]; if constexpr (PERCH) av[e] = an[e]; }
+                v = vn; beta = bn; ah = ahn; kq = kqn;
+            }
         }
     }
 #pragma unroll
