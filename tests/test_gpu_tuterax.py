@@ -379,6 +379,49 @@ def test_other_sizes(pkg, tmp_path, name, cfg):
     assert close(got, want)
 
 
+@pytest.mark.parametrize("seed", [101, 102, 103, 104])
+def test_configurations_drawn_at_random(pkg, tmp_path, seed):
+    """Five to nine layers of any kind in any order with sizes drawn from lists (head counts 1 - 32, head sizes 16 - 128, two to four taps, ranks, with and
+    without feed-forward, cap and key / query rotation): a 400-token request in portions beside a short one that comes and goes in the same batches."""
+    rng = np.random.default_rng(seed)
+
+    def pick(xs):
+        return xs[int(rng.integers(0, len(xs)))]
+
+    layers = []
+    for _ in range(int(rng.integers(5, 10))):
+        kind = pick(["attention", "delta", "channel_delta"])
+        mlp = S.dense(pick([72, 200, 328])) if rng.random() < 0.6 else None
+        if kind == "attention":
+            G = pick([1, 2, 4]); H = G * pick([1, 2, 4, 8]); D = pick([16, 32, 64, 128])
+            layers.append(S.attention(heads=H, kv_heads=G, dim=D, vdim=pick([16, 32, 64, 96]), rot_dims=pick([0, 8, 16, D]), base=pick([1000.0, 30000.0, 500000.0]),
+                                      scale=pick([0.1, 0.2, 0.3]), softcap=pick([0, 10.0, 25.0, 50.0]), mlp=mlp))
+        else:
+            G = pick([1, 2, 3]); H = G * pick([1, 2, 4])
+            kw = dict(heads=H, kv_heads=G, dim=pick([16, 32, 64, 128]), vdim=pick([16, 32, 64, 128]), conv=pick([2, 3, 4]), mlp=mlp)
+            layers.append(S.delta(**kw) if kind == "delta" else S.channel_delta(ranks=(pick([8, 24, 32]), pick([8, 24, 40])), **kw))
+    cfg = S.config(layers, width=pick([136, 200, 320]), vocab=pick([300, 1021]), eps=pick([1e-5, 1e-6]), embed_scale=pick([1.0, 4.0, 12.0]))
+    rig = Rig(pkg, tmp_path / "drawn", cfg, seed=seed)
+    V = cfg["vocab"]
+    long, short = toks(400, V, seed), toks(23, V, seed + 1)
+    c = rig.ctx(n_ctx=512, n_ubatch=128)
+    got_long, got_short, at = [], [], 0
+    for k, n in enumerate([150, 1, 2, 97, 1, 1, 64, 84]):
+        tk, ps, sq = long[at:at + n], list(range(at, at + n)), [0] * n
+        if k in (1, 5):                                          # the short request rides along, whole, and leaves again
+            tk, ps, sq = tk + short, ps + list(range(len(short))), sq + [1] * len(short)
+        assert c.decode(tk, ps, seq=sq, logits=[1] * len(tk)) == 0
+        rows = np.stack([c.logits(i) for i in range(len(tk))])
+        got_long.append(rows[:n])
+        if k in (1, 5):
+            got_short.append(rows[n:])
+            assert c.kv_seq_rm(1, -1, -1)
+        at += n
+    assert close(np.concatenate(got_long), rig.ref(long))
+    for g in got_short:
+        assert close(g, rig.ref(short))
+
+
 def test_wide_outputs_with_one_to_four_rows(pkg, tmp_path):
     """A head with thousands of output columns (the embedding table read as the output head) and one to four rows takes the four-weight-rows-per-wave form
     of the weight-stream kernel: portions of 1, 3 and 4 tokens in both precisions (up to 16 rows the activations stay f32 in either)."""
