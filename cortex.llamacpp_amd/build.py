@@ -54,7 +54,8 @@ def _hipcc() -> str:
     return "hipcc"
 
 
-def build(force: bool = False, verbose: bool = False) -> str:
+def build(force: bool = False, verbose: bool = False, server: bool = True) -> str:
+    """Compiles what changed and links the library; server=False leaves the HTTP host and the row-split worker (plain C++ programs beside it) unbuilt."""
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     os.makedirs(os.path.dirname(LIB), exist_ok=True)
@@ -93,7 +94,8 @@ def build(force: bool = False, verbose: bool = False) -> str:
             raise RuntimeError(f"link failed:\n{r.stderr}")
         with open(stamp, "w") as f:
             f.write(want)
-    build_server(force)
+    if server:
+        build_server(force)
     return LIB
 
 
