@@ -42,6 +42,7 @@ struct NvxLayer {
     int heads = 0, dim = 0, vdim = 0, rot = 0, kv_rank = 0, q_rank = 0, window = 0, rot_dims = 0;
     float scale = 1.0f, rot_mscale = 1.0f, gate_cap = 1.0f;
     float *rot_freq = nullptr;      // [rot_dims / 2] radians per position
+    // norm weights in front of the mixer / the feed-forward (norm1, norm2; nullptr: the sublayer reads the stream itself) and behind them (norm1b, norm2b)
     float *norm1 = nullptr, *norm1b = nullptr, *norm2 = nullptr, *norm2b = nullptr;
     // latent attention: down = [dq ; dkv] rows, uk_t = per head [kv_rank][dim] (W_uk transposed inside each head), uv = per head [vdim][kv_rank]
     BfMat down, uq, uk_t, uv, o;
