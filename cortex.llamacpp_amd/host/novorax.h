@@ -1,4 +1,4 @@
-// novorax.h — the layer stack of the folder models (config.json + model.safetensors, bf16 weights) as this runtime holds it.  Two designs fill it.
+// novorax.h — the layer stack of the folder models (config.json + model.safetensors, bf16 weights) as this runtime holds it.  Three designs fill it.
 //
 // Novorax: a decoder whose layers each pick a token mixer (latent attention with a sliding window and a
 // softmax sink, or the mLSTM matrix-memory recurrence) and a feed-forward (dense relu^2, or experts chosen by a token-id table), norms on both sides of every
