@@ -10,6 +10,11 @@
 // key head in the rotate-half layout (entry i pairs with entry i + rot_dims / 2; the per-pair angle table comes from the host); the score multipliers (one
 // number for the layer, one per head) folded into the query; keys and values stored to the token's cache row.
 //
+// Optional per layer: a query multiplier that grows with the logarithm of the position (in steps of `every` positions); a learned bias per (distance bucket,
+// head) added to the score behind the soft cap (the host hands over the distance -> bucket table); cells at the first `keep_first` positions that stay seen
+// outside the window; the neighbour layout of the rotation (entry 2i with 2i + 1); several score maps per head over the same values - every (head, map) then
+// runs as a query head of its own with its own key head, and gq_maps_out joins two maps: a1 - lambda a2, unit RMS, a constant, an elementwise sigmoid gate.
+//
 // Turned values (optional): every value head is stored turned by its own position over all its entries, in the same half-and-half pairing; the weighted sum
 // of a row is turned back by the row's position - each term then carries the turn by (key position - query position), a relative position signal on the
 // value side.  The turn back happens where a row's result is finished: in the per-row kernel, in the merge of split scans, or in gq_unturn behind the tiled pass.
@@ -40,13 +45,14 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
     __shared__ float cs[2][GQ_MAX_D / 2];                       // cos / sin of the token's angle per pair: computed once, read by every head
     __shared__ float csv[2][GQ_MAX_D / 2];                      // the same for the value heads' pairs
     const int t = blockIdx.x, tid = threadIdx.x;
-    const int NQ = a.H * a.dim, NK = a.G * a.dim, NV = a.G * a.vdim, half = a.rot_dims >> 1;
+    const int GK = a.G * (a.maps > 1 ? a.maps : 1);             // key heads: one per (value head, map)
+    const int NQ = a.H * a.dim, NK = GK * a.dim, NV = a.G * a.vdim, half = a.rot_dims >> 1;
     const float *qr = a.p + (size_t)t * a.ld_p, *kr = qr + NQ, *vr = kr + NK;
     float inv_q = 1.0f, inv_k = 1.0f;
     const bool per_head = a.norm_per_head && a.wq_norm && a.wk_norm;
     if (per_head) {
         // sixteen lanes per head, queries then keys (q | k lie side by side in the row): every lane group's loads are on their way at once
-        for (int hh = tid >> 4; hh < a.H + a.G; hh += 16) {
+        for (int hh = tid >> 4; hh < a.H + GK; hh += 16) {
             const float *src = qr + (size_t)hh * a.dim;
             float ss = 0.0f;
             for (int i = tid & 15; i < a.dim; i += 16) { const float v = src[i]; ss = fmaf(v, v, ss); }
@@ -65,6 +71,8 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
         inv_k = 1.0f / sqrtf(gq_block_sum_256(ss, sh) / (float)NK + a.eps);
     }
     const float p = (float)a.tok_pos[t];
+    // (floor((p + 1) / every) as an integer division: exact)
+    const float q_temp = a.q_temp_every > 0 ? 1.0f + a.q_temp_coef * logf((float)((a.tok_pos[t] + 1) / a.q_temp_every) + 1.0f) : 1.0f;
     if (tid < half) sincosf(p * a.rot_freq[tid], &cs[1][tid], &cs[0][tid]);
     const int vhalf = a.v_rot_freq ? a.vdim >> 1 : 0;
     if (tid >= 128 && tid - 128 < vhalf) {                       // (the upper waves: beside the key / query table of the lower ones)
@@ -88,7 +96,13 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
         const float inv = per_head ? head_inv[i / a.dim] : isq ? inv_q : inv_k;
         const int wb = per_head ? 0 : b;                         // (a shared weight vector starts over with every head)
         float o;
-        if (d < a.rot_dims) {
+        if (d < a.rot_dims && a.rot_neighbours) {
+            const int j = d >> 1;
+            const float c = cs[0][j], s = cs[1][j];
+            float u = src[b + 2 * j] * inv, w = src[b + 2 * j + 1] * inv;
+            if (wn) { u *= wn[wb + 2 * j]; w *= wn[wb + 2 * j + 1]; }
+            o = (d & 1) == 0 ? u * c - w * s : w * c + u * s;
+        } else if (d < a.rot_dims) {
             const int j = d < half ? d : d - half;
             const float c = cs[0][j], s = cs[1][j];
             float u = src[b + j] * inv, w = src[b + j + half] * inv;
@@ -99,7 +113,7 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
             if (wn) o *= wn[wb + d];
         }
         if (isq) {
-            float m = a.q_scale;
+            float m = a.q_scale * q_temp;
             if (a.head_scale) m *= a.head_scale[e / a.dim];
             qo[e] = o * m;
         } else row[e] = o;
@@ -134,6 +148,38 @@ __global__ __launch_bounds__(256) void gq_unturn_kernel(GqAttnArgs a) {
     }
 }
 
+// where query head h (a (head, map) pair when a.maps > 1) finds its key head and its value head inside a cache row, and the row's length
+struct GqHeads { size_t row, koff, voff; };
+__device__ __forceinline__ GqHeads gq_heads(const GqAttnArgs &a, int h) {
+    const int maps = a.maps > 1 ? a.maps : 1, head = h / maps, map = h - head * maps, kvh = head / ((a.H / maps) / a.G);
+    GqHeads o;
+    o.row = (size_t)a.G * ((size_t)maps * a.dim + a.vdim);
+    o.koff = ((size_t)kvh * maps + map) * a.dim;
+    o.voff = (size_t)a.G * maps * a.dim + (size_t)kvh * a.vdim;
+    return o;
+}
+// the learned bias of head h at distance dist >= 0
+__device__ __forceinline__ float gq_rel_bias(const GqAttnArgs &a, int dist, int h) {
+    const int b = dist < a.n_dist ? a.dist_bucket[dist] : a.rel_rows - 1;
+    return a.rel[(size_t)b * a.H + h];
+}
+
+// y[t][h] = unit_rms(a1 - lambda a2) * out_mult * sigmoid(gate[t][h]) entry by entry; a1, a2 = the two maps' outputs of head h
+__global__ __launch_bounds__(64) void gq_maps_out_kernel(const float *att, int ld_att, const float *gate, int ld_gate, int VD, float lambda, float out_mult, float eps,
+                                                         float *y, int ld_y) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float *a1 = att + (size_t)t * ld_att + (size_t)(2 * h) * VD, *a2 = a1 + VD;
+    float ss = 0.0f;
+    for (int i = lane; i < VD; i += 64) { const float o = a1[i] - lambda * a2[i]; ss = fmaf(o, o, ss); }
+    ss = gq_wave_sum(ss);
+    const float inv = out_mult / sqrtf(ss / (float)VD + eps);
+    for (int i = lane; i < VD; i += 64) {
+        const float o = a1[i] - lambda * a2[i];
+        const float g = gate ? 1.0f / (1.0f + expf(-gate[(size_t)t * ld_gate + (size_t)h * VD + i])) : 1.0f;
+        y[(size_t)t * ld_y + (size_t)h * VD + i] = o * inv * g;
+    }
+}
+
 // One workgroup per (token, head), NW waves.  A wave works on four cells at a time: each 16-lane group owns one cell, its lanes hold elements
 // 64 j + 4 li .. + 3 of the key head and of the value head (16-byte loads) and the matching running sums; the next four cells of the wave are requested
 // before the current ones are used.  Every group keeps its own running maximum / sum / weighted value; groups, then waves, are merged at the end together
@@ -146,8 +192,8 @@ __global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
     float *qv = lds;                                            // [LP] (zero beyond dim)
     float *wm = lds + LP, *wl = wm + NW, *wacc = wl + NW;        // [NW], [NW], [NW][LP]
     const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, li = lane & 15;
-    const int kvh = h / (a.H / a.G);
-    const size_t L = (size_t)a.G * (D + VD), koff = (size_t)kvh * D, voff = (size_t)a.G * D + (size_t)kvh * VD;
+    const GqHeads hd = gq_heads(a, h);
+    const size_t L = hd.row, koff = hd.koff, voff = hd.voff;
     const int tpos = a.tok_pos[t];
     const uint64_t sbit = 1ull << (a.tok_seq[t] & 63);
     for (int i = tid; i < LP; i += blockDim.x) qv[i] = i < D ? a.q[(size_t)t * a.ld_q + (size_t)h * D + i] : 0.0f;
@@ -170,10 +216,11 @@ __global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
         c_lo += (int)blockIdx.z * per;
         c_hi = c_lo + per < c_hi ? c_lo + per : c_hi;
     }
-    const auto visible = [&](int c) {
+    const auto visible = [&](int c, int &dist) {
         if (c >= c_hi) return false;
         const int cp = a.cell_pos[c];
-        return cp >= 0 && cp <= tpos && (a.cell_seq[c] & sbit) != 0 && !(a.window > 0 && tpos - cp >= a.window);
+        dist = tpos - cp;
+        return cp >= 0 && cp <= tpos && (a.cell_seq[c] & sbit) != 0 && !(a.window > 0 && tpos - cp >= a.window && cp >= a.keep_first);
     };
     const auto fetch = [&](int c, bool vis, float (&dk)[NJ][4], float (&dv)[NJ][4]) {
         const float *kr = a.cache + (size_t)c * L + koff, *vr = a.cache + (size_t)c * L + voff;
@@ -195,12 +242,12 @@ __global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
             }
         }
     };
-    int c = c_lo + wave * 4 + g;
-    bool vis = visible(c);
+    int c = c_lo + wave * 4 + g, dist = 0, distn = 0;
+    bool vis = visible(c, dist);
     fetch(c, vis, ck, cv);
     for (int c0 = c_lo; c0 < c_hi; c0 += stride) {              // (uniform trip count: the shuffles below are executed by whole waves)
         const int cn = c + stride;
-        const bool visn = visible(cn);
+        const bool visn = visible(cn, distn);
         fetch(cn, visn, nk, nv);
         float dot = 0.0f;
 #pragma unroll
@@ -212,6 +259,7 @@ __global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
         for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);
         if (a.softcap > 0.0f) dot = a.softcap * tanhf(dot / a.softcap);
         if (vis) {
+            if (a.rel) dot += gq_rel_bias(a, dist, h);
             const float mn = fmaxf(m, dot), alpha = expf(m - mn), p = expf(dot - mn);   // (m = -inf at the group's first cell: alpha = 0)
             l = l * alpha + p;
 #pragma unroll
@@ -224,7 +272,7 @@ __global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
         for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int e = 0; e < 4; e++) { ck[j][e] = nk[j][e]; cv[j][e] = nv[j][e]; }
-        c = cn; vis = visn;
+        c = cn; vis = visn; dist = distn;
     }
     // the four groups of a wave -> one record per wave
     float M = fmaxf(m, __shfl_xor(m, 16, 64));
@@ -354,8 +402,9 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
     int *cpos = reinterpret_cast<int *>(cseq + GQT_B), *rpos = cpos + GQT_B, *rseq = rpos + BQ;
     __shared__ int red[4];
     const int D = a.dim, VD = a.vdim, tid = threadIdx.x, tq = tid >> 4, tc = tid & 15;
-    const int row0 = blockIdx.x * BQ, h = blockIdx.y, kvh = h / (a.H / a.G);
-    const size_t L = (size_t)a.G * (D + VD), koff = (size_t)kvh * D, voff = (size_t)a.G * D + (size_t)kvh * VD;
+    const int row0 = blockIdx.x * BQ, h = blockIdx.y;
+    const GqHeads hd = gq_heads(a, h);
+    const size_t L = hd.row, koff = hd.koff, voff = hd.voff;
     const int n_kv = *a.n_kv_dev;
     // the tile's rows: position and sequence of each; over the tile: first and last position, the union of sequences, the range of cells to walk
     int my_lo = 0x7fffffff, my_hi = 0, my_pmin = 0x7fffffff, my_pmax = -1;
@@ -403,7 +452,7 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
             int cp = -1; uint64_t cs = 0;
             if (c < c_end) { cp = a.cell_pos[c]; cs = a.cell_seq[c]; }
             cpos[tid] = cp; cseq[tid] = cs;
-            any = cp >= 0 && cp <= pmax && (cs & seqs) != 0 && !(a.window > 0 && pmin - cp >= a.window);
+            any = cp >= 0 && cp <= pmax && (cs & seqs) != 0 && !(a.window > 0 && pmin - cp >= a.window && cp >= a.keep_first);
         }
         if (!__syncthreads_or(any)) continue;
         // ---- S = Q K^T
@@ -457,8 +506,11 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int cp = cpos[tc + 16 * j];
-                vis[j] = cp >= 0 && cp <= rp && (cseq[tc + 16 * j] & rbit) != 0 && !(a.window > 0 && rp - cp >= a.window);
-                if (vis[j]) bm = fmaxf(bm, s[i][j]);
+                vis[j] = cp >= 0 && cp <= rp && (cseq[tc + 16 * j] & rbit) != 0 && !(a.window > 0 && rp - cp >= a.window && cp >= a.keep_first);
+                if (vis[j]) {
+                    if (a.rel) s[i][j] += gq_rel_bias(a, rp - cp, h);
+                    bm = fmaxf(bm, s[i][j]);
+                }
             }
 #pragma unroll
             for (int of = 8; of > 0; of >>= 1) bm = fmaxf(bm, __shfl_xor(bm, of, 64));
@@ -570,18 +622,30 @@ static hipError_t launch_gq_attn_tile(const GqAttnArgs &a, hipStream_t st) {
 
 bool gq_attn_shape_ok(int H, int G, int dim, int vdim) { return H >= 1 && G >= 1 && H % G == 0 && dim >= 1 && vdim >= 1 && dim <= GQ_MAX_D && vdim <= GQ_MAX_D; }
 
+hipError_t launch_gq_maps_out(const float *att, int ld_att, const float *gate, int ld_gate, int T, int H, int vdim, float lambda, float out_mult, float eps,
+                              float *y, int ld_y, hipStream_t st) {
+    if (T <= 0) return hipSuccess;
+    if (H < 1 || vdim < 1 || !att || !y) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(gq_maps_out_kernel, dim3((unsigned)T, (unsigned)H), dim3(64), 0, st, att, ld_att, gate, ld_gate, vdim, lambda, out_mult, eps, y, ld_y);
+    return hipGetLastError();
+}
+
 hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
     if (a.rot_dims < 0 || a.rot_dims > a.dim || a.rot_dims > GQ_MAX_D || (a.rot_dims & 1) || (a.rot_dims > 0 && !a.rot_freq)) return hipErrorInvalidValue;
     if (a.v_rot_freq && ((a.vdim & 1) || a.vdim > GQ_MAX_D || !a.v_cs)) return hipErrorInvalidValue;
-    if (a.norm_per_head && (size_t)(a.H + a.G) * sizeof(float) > 32 * 1024) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(gq_prep_kernel, dim3((unsigned)a.T), dim3(256), a.norm_per_head ? (size_t)(a.H + a.G) * sizeof(float) : 0, st, a);
+    const int n_heads = a.H + a.G * (a.maps > 1 ? a.maps : 1);
+    if (a.maps > 1 && a.H % a.maps != 0) return hipErrorInvalidValue;
+    if (a.norm_per_head && (size_t)n_heads * sizeof(float) > 32 * 1024) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(gq_prep_kernel, dim3((unsigned)a.T), dim3(256), a.norm_per_head ? (size_t)n_heads * sizeof(float) : 0, st, a);
     return hipGetLastError();
 }
 
 hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
-    if (!gq_attn_shape_ok(a.H, a.G, a.dim, a.vdim) || (a.v_cs && (a.vdim & 1))) return hipErrorInvalidValue;
+    const int maps = a.maps > 1 ? a.maps : 1;
+    if (a.H % maps != 0 || !gq_attn_shape_ok(a.H / maps, a.G, a.dim, a.vdim) || (a.v_cs && (a.vdim & 1))) return hipErrorInvalidValue;
+    if (a.rel && (!a.dist_bucket || a.n_dist < 0 || a.rel_rows < 1)) return hipErrorInvalidValue;
     // batches: the tiled pass (16-byte loads everywhere: head sizes, strides and bases must allow them); a few rows: one workgroup per (row, head)
     const auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (a.T >= GQ_TILE_MIN_ROWS && (a.dim & 3) == 0 && (a.vdim & 3) == 0 && (a.ld_q & 3) == 0 && (a.ld_out & 3) == 0 && al16(a.q) && al16(a.out) && al16(a.cache)) {

@@ -262,7 +262,8 @@ hipError_t launch_moe_scatter_combine(float *x, const float *y, const float *w, 
 // Outer index z < nz, one of: plain strides (x_zs / w_zs / y_zs elements; per-head products); meta != nullptr: z is an expert, its rows of X and Y are
 // [meta[nz + z], + meta[z]) (launch_moe_group's counts | offsets; T = upper bound of any expert's rows); sel != nullptr: z is a (token, rank) pair - weight set
 // sel[z], row z / sel_div of X, row z of Y.
-enum { MMB_STORE = 0, MMB_RELU2 = 1, MMB_SILU_MUL = 2, MMB_GELU_MUL = 3 };   // y | relu(y)^2 | silu(W x) * (W2 x) | gelu_tanh(W x) * (W2 x)
+// y | relu(y)^2 | silu(W x) * (W2 x) | gelu_tanh(W x) * (W2 x) | g sigmoid(1.702 g) (u + 1) with g = min(W x, epi_limit), u = clamp(W2 x, -epi_limit, epi_limit)
+enum { MMB_STORE = 0, MMB_RELU2 = 1, MMB_SILU_MUL = 2, MMB_GELU_MUL = 3, MMB_CLAMP_SWIGLU = 4 };
 constexpr int MMB_VEC_ROWS = 16;                               // up to this many rows take the one-wave-per-column kernel
 struct MMBArgs {
     const float *x = nullptr; int ldx = 0;
@@ -270,6 +271,8 @@ struct MMBArgs {
     float *y = nullptr; int ldy = 0;
     int T = 0, N = 0, K = 0, epi = MMB_STORE, f32 = 0;
     float out_scale = 1.0f;                                    // multiplies every stored value (a model's logit scale)
+    float epi_limit = 0.0f;                                    // MMB_CLAMP_SWIGLU: the clamp
+    const float *bias = nullptr;                               // nullable, [N] f32: added to W x before the epilogue (the same vector for every outer index)
     int nz = 1; long long x_zs = 0, w_zs = 0, y_zs = 0;
     const int32_t *meta = nullptr;
     const int32_t *sel = nullptr; int sel_div = 1;
@@ -289,12 +292,21 @@ hipError_t launch_moe_uniform_combine(float *out, const float *y, const int32_t 
 // largest s, only experts of the `keep` best groups can be taken; the k best of them, weights s / (their sum + 1e-20) * scale.  ids / w: [T][k], best first.
 constexpr int MOE_ROUTE_MAX_EXPERTS = 8192;
 hipError_t launch_moe_route_groups(const float *z, int ld_z, int T, int E, int k, int n_group, int keep, float scale, int32_t *ids, float *w, hipStream_t st);
+// router with a selection bias (misc.hip): s = sigmoid(z[t][0 .. E)); the choice score of an expert is c = s + bias (bias nullable; c may be negative); the experts
+// form n_group equal groups of neighbours, a group scores as the sum of its two largest c (its only one if it holds one expert), only experts of the `keep`
+// best groups can be taken; the k open experts with the largest c, lowest index first on a tie; weights = their s as it is.  ids / w: [T][k], best first.
+hipError_t launch_moe_route_sigmoid_bias(const float *z, int ld_z, const float *bias, int T, int E, int k, int n_group, int keep, int32_t *ids, float *w, hipStream_t st);
+// out[t][:] = sum_j w[t][j] * y[row(t, j)] [+ sigmoid(sg[t * ld_sg]) * b[t]]: the routed experts' weighted sum (rank order) and an always-on expert b (nullable)
+// behind its one-number gate; row(t, j) = slot_of[t * k + j], or t * k + j without a grouping
+hipError_t launch_moe_weighted_combine(float *out, const float *y, const float *w, const int32_t *slot_of, const float *b, const float *sg, int ld_sg, int T, int E, int k, hipStream_t st);
 // x[t][:] += m * (a[t] + b[t] + sum_j w[t][j] * y[row(t, j)]): the close of a block whose mixer (a), always-on expert (b, nullable) and routed experts (y; k = 0:
 // none) all read the same normed input; row(t, j) = slot_of[t * k + j], or t * k + j without a grouping
 hipError_t launch_block_combine(float *x, const float *a, const float *b, const float *y, const float *w, const int32_t *slot_of, int T, int E, int k, float m, hipStream_t st);
 
 // ---------------------------------------------------------------- grouped-query attention on f32 cache rows (gq_attn.hip)
 // cache row of a cell: [G key heads of dim | G value heads of vdim] f32.  Query head h reads key / value head h / (H / G).
+// maps = M > 1 (several score maps per head over the same values): the query rows are [H][M][dim], the key rows [G][M][dim] (the cache row holds G * M key
+// heads, then G value heads); the attention treats every (head, map) as a query head of its own - H * M outputs of vdim per token, which launch_gq_maps_out joins.
 struct GqPrepArgs {
     const float *p; int ld_p;              // [T][q: H*dim | k: G*dim | v: G*vdim | ...] projections of the batch
     int T, H, G, dim, vdim;
@@ -302,6 +314,9 @@ struct GqPrepArgs {
     int norm_per_head;                     // 1: the statistic is taken over each head's dim entries instead, and the weights are [dim], shared by the heads
     int rot_dims; const float *rot_freq;   // the first rot_dims entries of every q / k head turn, entry i with entry i + rot_dims / 2; [rot_dims / 2] radians per position
     float q_scale; const float *head_scale;      // the query is multiplied by q_scale * head_scale[h] (nullable): the score's constant factors
+    int maps;                              // score maps per head (0 or 1: one)
+    int rot_neighbours;                    // 1: entry 2i turns with entry 2i + 1 instead of entry i with entry i + rot_dims / 2
+    float q_temp_coef; int q_temp_every;   // q_temp_every > 0: the query at position p is also multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)
     const int32_t *tok_pos, *tok_cell;
     float *q; int ld_q;                    // [T][H*dim]: normed, turned, scaled queries
     float *cache;                          // [n_ctx][G*dim + G*vdim]
@@ -318,6 +333,11 @@ struct GqAttnArgs {
     const float *cache;
     const int32_t *cell_pos; const uint64_t *cell_seq; const int32_t *tok_pos, *tok_seq; const int32_t *n_kv_dev;
     int window;                            // cells at distance 0 .. window - 1 are seen; 0 = every earlier cell
+    int keep_first;                        // with a window: cells at positions below keep_first stay seen at any distance
+    int maps;                              // score maps per head (0 or 1: one); H counts (head, map) pairs, G the value heads
+    // nullable: a learned bias per (distance bucket, head) added to the score behind the soft cap: rel[bucket(d) * rel_heads + h], bucket(d) = dist_bucket[d]
+    // for d < n_dist, else rel_rows - 1
+    const float *rel; const int32_t *dist_bucket; int n_dist, rel_rows;
     const float *sink;                     // [H] or nullptr: a logit without key or value in the softmax denominator
     const float *gate; int ld_gate;        // nullable: head h's output is multiplied by sigmoid(gate[t * ld_gate + h])
     float softcap;                         // > 0: a score s becomes softcap * tanh(s / softcap) before the softmax
@@ -334,6 +354,9 @@ constexpr int GQ_TILE_MAX_SPLITS = 16;
 constexpr int GQ_TILE_MIN_ROWS = 32;     // batches from this many rows on take the LDS-tiled pass (64 rows x 64 cells per step) instead of one workgroup per (row, head)
 bool gq_attn_shape_ok(int H, int G, int dim, int vdim);
 hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st);
+// two score maps joined: y[t][h][:] = unit_rms(a1 - lambda * a2) * out_mult * sigmoid(gate[t * ld_gate + h * vdim + :]), a1 / a2 = att[t][2h], att[t][2h + 1]
+hipError_t launch_gq_maps_out(const float *att, int ld_att, const float *gate, int ld_gate, int T, int H, int vdim, float lambda, float out_mult, float eps,
+                              float *y, int ld_y, hipStream_t st);
 
 // ---------------------------------------------------------------- latent attention (latent_attn.hip)
 // cache row of a cell: [kv_rank normed latent | rot rotated shared key part] f32.  rot_freq: [rot_dims / 2] angles per position (host-made, YaRN blend
@@ -387,6 +410,23 @@ enum { MLSTM_GATE_SIGMOID = 0, MLSTM_GATE_SILU = 1 };
 hipError_t launch_mlstm_out(const float *o, int ld_o, const float *p, int ld_p, int off_g, const float *w, int T, int H, int VD, float eps, float *y, int ld_y,
                             hipStream_t st, int w_stride = -1, int gate = MLSTM_GATE_SIGMOID);
 hipError_t launch_mlstm_state_reset(float *S, size_t n_s, float *n, size_t n_n, float *m, size_t n_m, hipStream_t st);   // S = 0, n = 0, m = 0
+
+// ---------------------------------------------------------------- retention (retention.hip)
+// Linear attention with one fixed decay per head and no softmax: per head a state S [D][VD] f32 per sequence slot;  S <- decay S + k v^T;  o = S^T q.
+// The first rot_dims entries of every q / k head turn by the token's position (entry i with entry i + rot_dims / 2), k is multiplied by k_scale behind the turn.
+struct RetentionArgs {
+    const float *p; int ld_p;              // [T][q: H*D | k: H*D | v: H*VD | ...] projections of the batch
+    float *o; int ld_o;                    // [T][H][VD] outputs (before the per-head unit norm)
+    int H, D, VD;
+    const float *decay;                    // [H]
+    int rot_dims; const float *rot_freq;   // [rot_dims / 2] radians per position
+    float k_scale;
+    const int32_t *tok_pos;
+    float *S;                              // [slot][H][D][VD]
+    const int32_t *seg_start, *seg_len, *seg_slot; int n_seg;   // runs of consecutive batch rows of one sequence each; no slot twice in a launch
+};
+bool retention_shape_ok(int D, int VD);
+hipError_t launch_retention_scan(const RetentionArgs &a, hipStream_t st);
 
 // ---------------------------------------------------------------- gated delta rule (delta_rule.hip)
 // Per head a state matrix S [D][VD], f32, one per sequence slot.  For a token with unit-length key k, unit-length query q / sqrt(D), value v, write strength

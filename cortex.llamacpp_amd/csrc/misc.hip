@@ -612,6 +612,80 @@ hipError_t launch_moe_route_groups(const float *z, int ld_z, int T, int E, int k
     return hipGetLastError();
 }
 
+// Router with a selection bias: one wave per token.  s = sigmoid(z); the choice score c = s + bias decides who is taken, the weight of a taken expert is its s.
+// Groups of `per` neighbouring experts score as the sum of their two largest c; the experts of all but the `keep` best groups are closed (c = -inf: choice
+// scores may be negative, so nothing else can stand for "closed").  Ties go to the lower index.
+__global__ __launch_bounds__(64) void moe_route_sigmoid_bias_kernel(const float *z, int ld_z, const float *bias, int E, int k, int n_group, int keep, int32_t *ids, float *w) {
+    extern __shared__ float rl[];
+    float *c = rl, *gs = rl + E;                                // [E] choice scores (taken or closed: -inf), [n_group] group scores (a kept group's becomes -inf)
+    int *ti = reinterpret_cast<int *>(gs + n_group);            // [k] taken experts
+    const int t = blockIdx.x, lane = threadIdx.x, per = E / n_group;
+    const float *zr = z + (size_t)t * ld_z;
+    for (int e = lane; e < E; e += 64) c[e] = 1.0f / (1.0f + expf(-zr[e])) + (bias ? bias[e] : 0.0f);
+    __syncthreads();
+    const auto arg_best = [&](const float *v, int n) {
+        float bv = -INFINITY; int bi = n;
+        for (int i = lane; i < n; i += 64) if (v[i] > bv) { bv = v[i]; bi = i; }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64); const int oi = __shfl_xor(bi, o, 64);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        return bi;
+    };
+    if (n_group > 1 && keep < n_group) {
+        for (int gi = lane; gi < n_group; gi += 64) {
+            float b1 = -INFINITY, b2 = -INFINITY;
+            for (int e = gi * per; e < (gi + 1) * per; e++) {
+                const float x = c[e];
+                if (x > b1) { b2 = b1; b1 = x; } else if (x > b2) b2 = x;
+            }
+            gs[gi] = per > 1 ? b1 + b2 : b1;
+        }
+        __syncthreads();
+        for (int r = 0; r < keep; r++) {
+            const int gi = arg_best(gs, n_group);
+            __syncthreads();
+            if (lane == 0 && gi < n_group) gs[gi] = -INFINITY;
+            __syncthreads();
+        }
+        for (int e = lane; e < E; e += 64) if (gs[e / per] != -INFINITY) c[e] = -INFINITY;
+        __syncthreads();
+    }
+    for (int r = 0; r < k; r++) {
+        int ei = arg_best(c, E);
+        if (ei >= E) ei = 0;                                     // (fewer open experts than k: refused by the launcher)
+        __syncthreads();
+        if (lane == 0) { ti[r] = ei; c[ei] = -INFINITY; }
+        __syncthreads();
+    }
+    for (int r = lane; r < k; r += 64) { ids[(size_t)t * k + r] = ti[r]; w[(size_t)t * k + r] = 1.0f / (1.0f + expf(-zr[ti[r]])); }
+}
+hipError_t launch_moe_route_sigmoid_bias(const float *z, int ld_z, const float *bias, int T, int E, int k, int n_group, int keep, int32_t *ids, float *w, hipStream_t st) {
+    if (T <= 0) return hipSuccess;
+    if (E < 1 || E > MOE_ROUTE_MAX_EXPERTS || k < 1 || k > E || n_group < 1 || E % n_group != 0 || keep < 1 || keep > n_group) return hipErrorInvalidValue;
+    if ((long long)keep * (E / n_group) < k) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(moe_route_sigmoid_bias_kernel, dim3((unsigned)T), dim3(64), (size_t)(E + n_group + k) * sizeof(float), st, z, ld_z, bias, E, k, n_group, keep, ids, w);
+    return hipGetLastError();
+}
+
+// out[t][d] = sum_j w[t][j] * y[row(t, j)][d] (rank order) + sigmoid(sg[t * ld_sg]) * b[t][d]
+__global__ void moe_weighted_combine_kernel(float *out, const float *y, const float *w, const int32_t *slot_of, const float *b, const float *sg, int ld_sg, int T, int E, int k) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)T * E) return;
+    const int t = (int)(i / E), d = (int)(i - (int64_t)t * E);
+    float o = 0.0f;
+    for (int j = 0; j < k; j++) o += y[(size_t)(slot_of ? slot_of[(size_t)t * k + j] : t * k + j) * E + d] * w[(size_t)t * k + j];
+    if (b) o += (sg ? 1.0f / (1.0f + expf(-sg[(size_t)t * ld_sg])) : 1.0f) * b[i];
+    out[i] = o;
+}
+hipError_t launch_moe_weighted_combine(float *out, const float *y, const float *w, const int32_t *slot_of, const float *b, const float *sg, int ld_sg, int T, int E, int k, hipStream_t st) {
+    if ((int64_t)T * E <= 0) return hipSuccess;
+    if (k > 0 && (!y || !w)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(moe_weighted_combine_kernel, dim3((unsigned)(((int64_t)T * E + 255) / 256)), dim3(256), 0, st, out, y, w, slot_of, b, sg, ld_sg, T, E, k);
+    return hipGetLastError();
+}
+
 // The close of a block whose sublayers all read one normed input: x[t][d] += m * (a[t][d] + b[t][d] + sum_j w[t][j] * y[row(t, j)][d]); a = the mixer's output,
 // b = an always-on expert's (nullable), y = the routed experts' rows (row(t, j) = slot_of[t * k + j], or t * k + j without a grouping; k = 0: none), added in
 // rank order.

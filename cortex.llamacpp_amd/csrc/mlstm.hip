@@ -9,7 +9,7 @@
 // one sequence segment: lane = column, the 8 or 16 waves split the dim rows (each thread keeps its rows of its column - and of n - in registers), the per-token
 // partial sums of S^T q and n . q cross the waves through LDS.  A segment is a run of consecutive rows of the batch that belong to one sequence: a prompt,
 // a portion of one, or a single decoded token - the same code, started from the slot's state and ending with the state written back.
-// mlstm_out: per head, the output divided by its root mean square, times the mixer's norm weight (per head and entry, or one vector shared by the heads), times
+// mlstm_out: per head, the output divided by its root mean square, times the mixer's norm weight (per head and entry, one vector shared by the heads, or none), times
 // sigmoid - or silu - of the output gate's pre-activation.  The delta-rule mixers close with the same launch.
 #include "kernels.h"
 
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(64) void mlstm_out_kernel(const float *o, int ld_o,
     for (int i = lane; i < VD; i += 64) {
         const float g = p[(size_t)t * ld_p + off_g + h * VD + i];
         const float sg = 1.0f / (1.0f + expf(-g));
-        y[(size_t)t * ld_y + (size_t)h * VD + i] = orow[i] * inv * w[h * w_stride + i] * (gate == MLSTM_GATE_SILU ? g * sg : sg);
+        y[(size_t)t * ld_y + (size_t)h * VD + i] = orow[i] * inv * (w ? w[h * w_stride + i] : 1.0f) * (gate == MLSTM_GATE_SILU ? g * sg : sg);
     }
 }
 

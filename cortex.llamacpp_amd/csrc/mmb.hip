@@ -13,7 +13,8 @@
 //                 read K-contiguous straight into the matrix-core register layout (lane = (row, k-group of 8)).
 //   * mmb_f32   - batches in f32 mode (and every shape the other two refuse): LDS-tiled, v_fma_f32 only - products of an f32 activation and a bf16 weight
 //                 widened exactly, no reduced-precision matrix mode anywhere.
-// Epilogues: store | relu(y)^2 | silu(W x) * (W2 x) | gelu_tanh(W x) * (W2 x) (the gated ones: two weight sets, one pass over the activations).
+// Epilogues: store | relu(y)^2 | silu(W x) * (W2 x) | gelu_tanh(W x) * (W2 x) | g sigmoid(1.702 g) (u + 1) with g = W x capped from above and u = W2 x clamped
+// to +- the same limit (the gated ones: two weight sets, one pass over the activations).  An optional f32 bias per output column joins W x before the epilogue.
 #include "kernels.h"
 
 namespace mi355 {
@@ -33,7 +34,11 @@ __device__ __forceinline__ unsigned short f2bf(float f) {                       
     u += 0x7fffu + ((u >> 16) & 1u);
     return (unsigned short)(u >> 16);
 }
-__device__ __forceinline__ float epi_apply(int epi, float a, float b) {
+__device__ __forceinline__ float epi_apply(int epi, float a, float b, float lim = 0.0f) {
+    if (epi == MMB_CLAMP_SWIGLU) {
+        const float g = fminf(a, lim), u = fminf(fmaxf(b, -lim), lim);
+        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    }
     if (epi == MMB_RELU2) { const float r = a > 0.0f ? a : 0.0f; return r * r; }
     if (epi == MMB_SILU_MUL) return a / (1.0f + expf(-a)) * b;
     if (epi == MMB_GELU_MUL) return 0.5f * a * (1.0f + tanhf(0.7978845608028654f * (a + 0.044715f * a * a * a))) * b;   // the tanh form of gelu; sqrt(2 / pi)
@@ -126,7 +131,7 @@ __global__ __launch_bounds__(256) void mmb_vec_rows_kernel(MMBArgs a) {
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) { s1 += __shfl_xor(s1, o, 64); s2 += __shfl_xor(s2, o, 64); }
             if (pn) { s1 *= inv; s2 *= inv; }
-            if (lane == 0 && n0 + r < a.N) v.y[(size_t)i * a.ldy + n0 + r] = epi_apply(a.epi, s1, s2) * a.out_scale;
+            if (lane == 0 && n0 + r < a.N) v.y[(size_t)i * a.ldy + n0 + r] = epi_apply(a.epi, a.bias ? s1 + a.bias[n0 + r] : s1, s2, a.epi_limit) * a.out_scale;
         }
     }
 }
@@ -195,7 +200,7 @@ __global__ __launch_bounds__(256) void mmb_vec_kernel(MMBArgs a) {
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) { s += __shfl_xor(s, o, 64); s2 += __shfl_xor(s2, o, 64); q += __shfl_xor(q, o, 64); }
             if (pn) { const float inv = 1.0f / sqrtf(q / (float)a.K + a.pn_eps); s *= inv; s2 *= inv; }
-            if (lane == 0) v.y[(size_t)(t0 + i) * a.ldy + n] = epi_apply(a.epi, s, s2) * a.out_scale;
+            if (lane == 0) v.y[(size_t)(t0 + i) * a.ldy + n] = epi_apply(a.epi, a.bias ? s + a.bias[n] : s, s2, a.epi_limit) * a.out_scale;
         }
     }
 }
@@ -256,7 +261,7 @@ __global__ __launch_bounds__(256) void mmb_f32_kernel(MMBArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int n = n0 + tx * 4 + j;
-            if (n < a.N) v.y[(size_t)t * a.ldy + n] = epi_apply(a.epi, acc[i][j], acc2[i][j]) * a.out_scale;
+            if (n < a.N) v.y[(size_t)t * a.ldy + n] = epi_apply(a.epi, a.bias ? acc[i][j] + a.bias[n] : acc[i][j], acc2[i][j], a.epi_limit) * a.out_scale;
         }
     }
 }
@@ -341,7 +346,7 @@ __global__ __launch_bounds__(256) void mmb_mfma_kernel(MMBArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int n = n0 + 32 * i + (r & 3) + 8 * (r >> 2) + 4 * kg;
-                if (n < a.N) v.y[(size_t)t * a.ldy + n] = epi_apply(a.epi, acc[i][j][r], GATED ? acc2[i][j][r] : 0.0f) * a.out_scale;
+                if (n < a.N) v.y[(size_t)t * a.ldy + n] = epi_apply(a.epi, a.bias ? acc[i][j][r] + a.bias[n] : acc[i][j][r], GATED ? acc2[i][j][r] : 0.0f, a.epi_limit) * a.out_scale;
             }
         }
 }
@@ -350,7 +355,7 @@ __global__ __launch_bounds__(256) void mmb_mfma_kernel(MMBArgs a) {
 
 hipError_t launch_mmb(const MMBArgs &a, hipStream_t st) {
     if (a.T <= 0 || a.N <= 0 || a.nz <= 0) return hipSuccess;
-    const bool gated = a.epi == MMB_SILU_MUL || a.epi == MMB_GELU_MUL;
+    const bool gated = a.epi == MMB_SILU_MUL || a.epi == MMB_GELU_MUL || a.epi == MMB_CLAMP_SWIGLU;
     if (a.K <= 0 || !a.x || !a.w || !a.y || (gated && !a.w2)) return hipErrorInvalidValue;
     const auto al = [](const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) == 0; };
     // 16-byte loads of both operands: every row start and every stride on a 16-byte boundary

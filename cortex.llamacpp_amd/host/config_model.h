@@ -1,6 +1,6 @@
 // config_model.h — what the loaders of the folder models (config.json + model.safetensors, bf16 weights) share: reading the configuration, checking every
 // tensor against it on the way to the device, and laying out the order of layer runs with its looped span.  One loader per design (novorax.cc, fidepel.cc,
-// tuterax.cc);
+// tuterax.cc, dinilorn.cc);
 // config_model_load picks it by the configuration's "architecture".
 #pragma once
 
@@ -131,9 +131,13 @@ bool cfg_layer_runs(const Json &loop, int n_layer, std::string &err, int &times_
     return true;
 }
 
+// from this many (token, rank) pairs on a routed feed-forward groups the pairs by expert and runs every expert's rows as one batch (fidepel.cc)
+bool nvx_routed_as_groups(const NvxLayer &L, int T);
+
 // the designs' loaders: cfg is the parsed config.json of `dir`, ld has model.safetensors open and ld.m set
 Model *novorax_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, std::string &err, int &status);
 Model *fidepel_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, std::string &err, int &status);
 Model *tuterax_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, std::string &err, int &status);
+Model *dinilorn_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, std::string &err, int &status);
 
 }  // namespace mi355

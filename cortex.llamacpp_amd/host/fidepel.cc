@@ -157,50 +157,60 @@ Model *fidepel_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, st
 // ------------------------------------------------------------------------------------------ the block
 // from this many (token, rank) pairs on, the pairs are grouped by expert and every expert runs its rows as one batch (launch_moe_group holds the pair list in
 // LDS and serves up to 64 experts); fewer pairs read their experts' rows directly
-static bool routed_as_groups(const NvxLayer &L, int T) {
+bool nvx_routed_as_groups(const NvxLayer &L, int T) {
     return L.ff_kind == NVX_FF_ROUTED && T * L.top > 32 && L.n_expert <= 64 && (size_t)T * L.top * 4 <= 60 * 1024;
 }
 
-// behind the block projection (nvx_a_): queries prepared, keys and values stored, attention, output projection -> nvx_y_
+// behind the block projection (nvx_a_): queries prepared, keys and values stored, attention, output projection -> nvx_y_.  With several score maps per head
+// every (head, map) pair runs as a query head of its own; launch_gq_maps_out joins the maps in front of the output projection.
 hipError_t Context::nvx_gq_attention(const NvxLayer &L, const NvxRun &r, int T) {
     const NovoraxModel &M = *model->nvx;
-    const int W = M.width, H = L.heads, G = L.kv_heads, LD_P = L.proj.N;
+    const int W = M.width, G = L.kv_heads, LD_P = L.proj.N, maps = L.maps > 1 ? L.maps : 1;
+    const int H = L.heads * maps;                               // query heads as the kernels count them
     float *cache = nvx_cache_[(size_t)r.plane];
     GqPrepArgs pa{};
     pa.p = nvx_a_; pa.ld_p = LD_P; pa.T = T; pa.H = H; pa.G = G; pa.dim = L.dim; pa.vdim = L.vdim;
     pa.wq_norm = L.q_norm; pa.wk_norm = L.k_norm; pa.eps = M.eps; pa.rot_dims = L.rot_dims; pa.rot_freq = L.rot_freq;
     pa.norm_per_head = L.qk_norm_per_head ? 1 : 0; pa.v_rot_freq = L.v_rot_freq; pa.v_cs = L.v_rot_freq ? nvx_vcs_ : nullptr;
     pa.q_scale = L.scale; pa.head_scale = L.head_scale; pa.tok_pos = d_pos_; pa.tok_cell = d_cell_;
+    pa.maps = maps; pa.rot_neighbours = L.rot_neighbours ? 1 : 0; pa.q_temp_coef = L.q_temp_coef; pa.q_temp_every = L.q_temp_every;
     pa.q = nvx_q_; pa.ld_q = H * L.dim; pa.cache = cache;
     FDP_TRY(launch_gq_prep(pa, stream_));
     GqAttnArgs aa{};
-    aa.q = nvx_q_; aa.ld_q = H * L.dim; aa.out = nvx_att_; aa.ld_out = H * L.vdim; aa.T = T; aa.H = H; aa.G = G; aa.dim = L.dim; aa.vdim = L.vdim;
+    aa.q = nvx_q_; aa.ld_q = H * L.dim; aa.out = maps > 1 ? nvx_o_ : nvx_att_; aa.ld_out = H * L.vdim; aa.T = T; aa.H = H; aa.G = G; aa.dim = L.dim; aa.vdim = L.vdim;
+    aa.maps = maps; aa.keep_first = L.keep_first; aa.rel = L.rel; aa.dist_bucket = L.dist_bucket; aa.n_dist = L.n_dist; aa.rel_rows = L.rel_rows;
     aa.cache = cache; aa.cell_pos = d_cell_pos_; aa.cell_seq = d_cell_seq_; aa.tok_pos = d_pos_; aa.tok_seq = d_seq_; aa.n_kv_dev = d_nkv_;
-    aa.window = L.window; aa.sink = L.sink; aa.gate = L.off_gate >= 0 ? nvx_a_ + L.off_gate : nullptr; aa.ld_gate = LD_P;
+    aa.window = L.window; aa.sink = L.sink; aa.gate = L.off_gate >= 0 && !L.gate_per_entry ? nvx_a_ + L.off_gate : nullptr; aa.ld_gate = LD_P;
     aa.softcap = L.softcap; aa.v_cs = L.v_rot_freq ? nvx_vcs_ : nullptr;
     aa.tok_hi = d_seg_ + 3 * (size_t)cp.n_ubatch;
-    aa.tok_lo = M.max_window > 0 ? d_seg_ + 4 * (size_t)cp.n_ubatch : nullptr;
+    aa.tok_lo = M.max_window > 0 && L.window > 0 ? d_seg_ + 4 * (size_t)cp.n_ubatch : nullptr;
     aa.part = nvx_part_; aa.part_floats = nvx_part_floats_; aa.n_kv_hint = n_kv_;
     aa.splits = (long long)T * H <= LATENT_ATTN_SPLIT_MAX_PAIRS ? LATENT_ATTN_SPLITS : 1;
     FDP_TRY(launch_gq_attn(aa, stream_));
-    FDP_TRY(nvx_linear(L.o, nvx_att_, H * L.vdim, T, nvx_y_, W));
+    if (maps == 2)
+        FDP_TRY(launch_gq_maps_out(nvx_o_, H * L.vdim, L.gate_per_entry ? nvx_a_ + L.off_gate : nullptr, LD_P, T, L.heads, L.vdim, L.map_lambda, L.map_mult, M.eps,
+                                   nvx_att_, L.heads * L.vdim, stream_));
+    else if (maps != 1) return hipErrorInvalidValue;
+    FDP_TRY(nvx_linear(L.o, nvx_att_, L.heads * L.vdim, T, nvx_y_, W, MMB_STORE, nullptr, 1.0f, nullptr, L.o_bias));
     prof_mark("gq_attention");
     return hipSuccess;
 }
 
-// the router's columns of the block projection -> experts and weights; the routed experts' rows end in nvx_yg_ (row(t, j): nvx_slot_ when grouped), the shared
-// expert's in nvx_ys_
-hipError_t Context::nvx_routed_experts(const NvxLayer &L, const float *h, const float *pn, int T) {
+// the router's logits -> experts and weights; the routed experts' rows end in nvx_yg_ (row(t, j): nvx_slot_ when grouped).  Experts are relu^2 (e_up alone)
+// or the clamped gated form (e_gate set)
+hipError_t Context::nvx_routed_experts(const NvxLayer &L, const float *h, const float *pn, int T, const float *z, int ld_z) {
     const NovoraxModel &M = *model->nvx;
     const int W = M.width, k = L.top, NE = L.n_expert, P = T * k;
-    FDP_TRY(launch_moe_route_groups(nvx_a_ + L.off_router, L.proj.N, T, NE, k, L.n_group, L.group_keep, L.router_scale, nvx_ids_, nvx_rw_, stream_));
+    if (L.route_kind == NVX_ROUTE_SIGMOID_BIAS) FDP_TRY(launch_moe_route_sigmoid_bias(z, ld_z, L.route_bias, T, NE, k, L.n_group, L.group_keep, nvx_ids_, nvx_rw_, stream_));
+    else FDP_TRY(launch_moe_route_groups(z, ld_z, T, NE, k, L.n_group, L.group_keep, L.router_scale, nvx_ids_, nvx_rw_, stream_));
     MMBArgs u;
     u.w = L.e_up.w; u.ldw = W; u.N = L.ff; u.K = W; u.epi = MMB_RELU2; u.f32 = cp.exact_f32 ? 1 : 0; u.w_zs = (long long)L.ff * W;
+    if (L.e_gate.w) { u.w = L.e_gate.w; u.w2 = L.e_up.w; u.epi = MMB_CLAMP_SWIGLU; u.epi_limit = L.expert_limit; }
     u.y = nvx_ff_; u.ldy = L.ff;
     MMBArgs d;
     d.w = L.e_down.w; d.ldw = L.ff; d.N = W; d.K = L.ff; d.f32 = u.f32; d.w_zs = (long long)W * L.ff;
     d.x = nvx_ff_; d.ldx = L.ff; d.y = nvx_yg_; d.ldy = W;
-    if (routed_as_groups(L, T)) {
+    if (nvx_routed_as_groups(L, T)) {
         // every expert sees its (token, rank) pairs as one batch of rows: counting sort by expert, gather, two grouped products
         FDP_TRY(launch_moe_group(nvx_ids_, T, k, NE, nvx_meta_, nvx_slot_, nvx_tokof_, stream_));
         FDP_TRY(launch_gather_rows_f32(h, nvx_tokof_, P, W, nvx_xg_, stream_));
@@ -220,7 +230,8 @@ hipError_t Context::nvx_routed_experts(const NvxLayer &L, const float *h, const 
 
 hipError_t Context::nvx_shared_expert(const NvxLayer &L, const float *h, const float *pn, int T) {
     const int W = model->nvx->width;
-    FDP_TRY(nvx_linear(L.s_up, h, W, T, nvx_sh_, L.shared_ff, MMB_RELU2, nullptr, 1.0f, pn));
+    if (L.s_gate.w) FDP_TRY(nvx_linear(L.s_gate, h, W, T, nvx_sh_, L.shared_ff, MMB_CLAMP_SWIGLU, &L.s_up, 1.0f, pn, nullptr, L.shared_limit));
+    else FDP_TRY(nvx_linear(L.s_up, h, W, T, nvx_sh_, L.shared_ff, MMB_RELU2, nullptr, 1.0f, pn));
     FDP_TRY(nvx_linear(L.s_down, nvx_sh_, L.shared_ff, T, nvx_ys_, W));
     prof_mark("shared_expert");
     return hipSuccess;
@@ -231,7 +242,7 @@ hipError_t Context::nvx_parallel_block(const NvxLayer &L, const NvxRun &r, int T
     const int W = M.width;
     // up to MMB_VEC_ROWS rows every reader norms the stream itself (no launch for the norm); batches norm once into xn_.  A grouped expert batch gathers
     // normed rows, so it needs xn_ too - with top >= 3 that starts below MMB_VEC_ROWS rows
-    const bool grouped = routed_as_groups(L, T);
+    const bool grouped = nvx_routed_as_groups(L, T);
     const bool fuse_norm = T <= MMB_VEC_ROWS && !grouped;
     const float *h = x_, *pn = L.norm1;
     if (!fuse_norm) {
@@ -253,7 +264,7 @@ hipError_t Context::nvx_parallel_block(const NvxLayer &L, const NvxRun &r, int T
         FDP_TRY(hipEventRecord(nvx_fork_ev_, main_stream));
         FDP_TRY(hipStreamWaitEvent(nvx_side_[0], nvx_fork_ev_, 0));
         stream_ = nvx_side_[0];
-        FDP_TRY(nvx_routed_experts(L, h, pn, T));
+        FDP_TRY(nvx_routed_experts(L, h, pn, T, nvx_a_ + L.off_router, L.proj.N));
         FDP_TRY(hipEventRecord(nvx_join_ev_[0], nvx_side_[0]));
         if (shared) {
             FDP_TRY(hipStreamWaitEvent(nvx_side_[1], nvx_fork_ev_, 0));
@@ -268,7 +279,7 @@ hipError_t Context::nvx_parallel_block(const NvxLayer &L, const NvxRun &r, int T
         FDP_TRY(hipStreamWaitEvent(main_stream, nvx_join_ev_[0], 0));
         if (shared) FDP_TRY(hipStreamWaitEvent(main_stream, nvx_join_ev_[1], 0));
     } else if (routed) {
-        FDP_TRY(nvx_routed_experts(L, h, pn, T));
+        FDP_TRY(nvx_routed_experts(L, h, pn, T, nvx_a_ + L.off_router, L.proj.N));
         if (shared) FDP_TRY(nvx_shared_expert(L, h, pn, T));
     }
     FDP_TRY(launch_block_combine(x_, nvx_y_, shared ? nvx_ys_ : nullptr, nvx_yg_, nvx_rw_, routed && grouped ? nvx_slot_ : nullptr, T, W,

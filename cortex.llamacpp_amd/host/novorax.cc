@@ -1,7 +1,7 @@
 // novorax.cc — the folder models (config.json + model.safetensors): the registry that picks a design's loader by "architecture", the Novorax loader, and what
 // every such design shares inside Context - buffers, cache planes and state slots, segment lists and scan bounds, the layer-run loop, the output head
 // (novorax.h describes the designs, runtime.h the context; the Fidepel loader and its block are in fidepel.cc, the Tuterax loader and the delta-rule mixer
-// in tuterax.cc).
+// in tuterax.cc, the Dinilorn loader, its retention mixer and its feed-forward in dinilorn.cc).
 //
 // The context's own machinery carries them: the cell table (find / free / sequence masks) addresses the attention layers' cache planes, the micro-batch staging
 // block brings tokens, positions, cells and sequence ids to the device, the sequence id is the slot of the recurrent state, logits / arg-max / top-k leave
@@ -49,6 +49,7 @@ Model *config_model_load(const std::string &dir, int main_gpu, std::string &err,
         {"Novorax", novorax_build},
         {"Fidepel", fidepel_build},
         {"Tuterax", tuterax_build},
+        {"Dinilorn", dinilorn_build},
     };
     status = -102;
     std::ifstream cf(dir + "/config.json");
@@ -257,9 +258,10 @@ Model *novorax_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, st
 static void nvx_state_sizes(const NvxLayer &L, size_t &s_sz, size_t &n_sz, size_t &m_sz) {
     s_sz = (size_t)L.heads * L.dim * L.vdim;
     if (L.type == NVX_MLSTM) { n_sz = (size_t)L.heads * L.dim; m_sz = (size_t)L.heads; }
+    else if (L.type == NVX_RETENTION) { n_sz = 0; m_sz = 0; }
     else { n_sz = (size_t)std::max(L.conv_taps - 1, 0) * (size_t)L.delta_channels(); m_sz = 0; }
 }
-static bool nvx_recurrent(const NvxLayer &L) { return L.type == NVX_MLSTM || L.type == NVX_DELTA; }
+static bool nvx_recurrent(const NvxLayer &L) { return L.type == NVX_MLSTM || L.type == NVX_DELTA || L.type == NVX_RETENTION; }
 
 bool Context::init_novorax(std::string &err) {
     const NovoraxModel &M = *model->nvx;
@@ -320,7 +322,7 @@ bool Context::init_novorax(std::string &err) {
         nvx_part_floats_ = (size_t)LATENT_ATTN_SPLIT_MAX_PAIRS * LATENT_ATTN_SPLITS * (size_t)(kr + 2);
         // grouped-query layers also cut the block chains of short prompt batches: records for up to 1024 rows x 4 runs of the widest layer
         for (const NvxLayer &L : M.layers)
-            if (L.type == NVX_GQ) nvx_part_floats_ = std::max(nvx_part_floats_, std::min<size_t>(T, 1024) * (size_t)L.heads * 4 * (size_t)(L.vdim + 2));
+            if (L.type == NVX_GQ) nvx_part_floats_ = std::max(nvx_part_floats_, std::min<size_t>(T, 1024) * (size_t)L.heads * (size_t)std::max(L.maps, 1) * 4 * (size_t)(L.vdim + 2));
         nvx_part_ = (float *)dalloc(nvx_part_floats_ * 4);
     }
     {
@@ -406,13 +408,13 @@ bool Context::nvx_stage_segments(int n, const int32_t *seq, const int32_t *pos, 
         int32_t *hi = h_seg_ + 3 * T, *lo = h_seg_ + 4 * T;
         int base[64], last_pos[64], first_pos[64], low[64];
         for (int s = 0; s < 64; s++) { base[s] = 0; last_pos[s] = -1; first_pos[s] = 0x7fffffff; low[s] = (int)cells_.size(); }
-        const int win = model->nvx->max_window;
+        const int win = model->nvx->max_window, kept = model->nvx->max_keep_first;   // (cells at the first `kept` positions stay in reach of a windowed layer)
         if (win > 0) {
             for (int i = 0; i < n; i++) first_pos[seq[i] & 63] = std::min(first_pos[seq[i] & 63], (int)pos[i]);
             for (size_t c = 0; c < cells_.size(); c++) {
                 if (cells_[c].pos < 0) continue;
                 uint64_t mk = cells_[c].seqs;
-                while (mk) { const int s = __builtin_ctzll(mk); mk &= mk - 1; if (first_pos[s] != 0x7fffffff && cells_[c].pos > first_pos[s] - win && (int)c < low[s]) low[s] = (int)c; }
+                while (mk) { const int s = __builtin_ctzll(mk); mk &= mk - 1; if (first_pos[s] != 0x7fffffff && (cells_[c].pos > first_pos[s] - win || cells_[c].pos < kept) && (int)c < low[s]) low[s] = (int)c; }
             }
         }
         for (int i = 0; i < n; i++) lo[i] = win > 0 ? low[seq[i] & 63] : 0;
@@ -452,7 +454,8 @@ bool Context::nvx_stage_segments(int n, const int32_t *seq, const int32_t *pos, 
 }
 
 // pn != nullptr: the rows of x are RMS-normed with weight (norm_off + pn) on the way in (few rows: inside the launch; batches: a norm launch into xn_ first)
-hipError_t Context::nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi, const BfMat *w2, float out_scale, const float *pn) {
+hipError_t Context::nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi, const BfMat *w2, float out_scale, const float *pn,
+                               const float *bias, float epi_limit) {
     MMBArgs a;
     if (pn && T > MMB_VEC_ROWS) {
         NVX_TRY(launch_rmsnorm_f32(x, ldx, pn, model->nvx->norm_off, nullptr, xn_, w.K, w.K, T, model->nvx->eps, stream_));
@@ -460,13 +463,14 @@ hipError_t Context::nvx_linear(const BfMat &w, const float *x, int ldx, int T, f
     }
     a.pn_w = pn; a.pn_off = model->nvx->norm_off; a.pn_eps = model->nvx->eps;
     a.x = x; a.ldx = ldx; a.w = w.w; a.w2 = w2 ? w2->w : nullptr; a.ldw = w.K; a.y = y; a.ldy = ldy;
-    a.T = T; a.N = w.N; a.K = w.K; a.epi = epi; a.f32 = cp.exact_f32 ? 1 : 0; a.out_scale = out_scale;
+    a.T = T; a.N = w.N; a.K = w.K; a.epi = epi; a.f32 = cp.exact_f32 ? 1 : 0; a.out_scale = out_scale; a.bias = bias; a.epi_limit = epi_limit;
     return launch_mmb(a, stream_);
 }
 
 hipError_t Context::nvx_feed_forward(const NvxLayer &L, int T) {
     const NovoraxModel &M = *model->nvx;
     const int W = M.width;
+    if (L.ff_kind == NVX_FF_ROUTED) return nvx_routed_feed_forward(L, T);
     if (L.ff_kind == NVX_FF_DENSE) {
         if (L.gate.w) NVX_TRY(nvx_linear(L.gate, x_, W, T, nvx_ff_, L.ff, MMB_GELU_MUL, &L.up, 1.0f, L.norm2));
         else NVX_TRY(nvx_linear(L.up, x_, W, T, nvx_ff_, L.ff, MMB_RELU2, nullptr, 1.0f, L.norm2));
@@ -512,12 +516,14 @@ hipError_t Context::run_layers_novorax(int T) {
     cur_T_ = T;
     NVX_TRY(launch_kv_meta_set(d_cell_pos_, d_cell_seq_, d_cell_, d_pos_, d_seqmask_, T, stream_));
     NVX_TRY(launch_get_rows(T_BF16, (const uint8_t *)M.embed.w, W, d_tok_, T, x_, stream_, M.embed_scale));
+    if (M.loop_add_embed) NVX_TRY(hipMemcpyAsync(nvx_x0_, x_, (size_t)T * W * 4, hipMemcpyDeviceToDevice, stream_));
     if (M.loop_in.w) NVX_TRY(hipMemcpy2DAsync(nvx_xcat_ + W, (size_t)2 * W * 4, x_, (size_t)W * 4, (size_t)W * 4, (size_t)T, hipMemcpyDeviceToDevice, stream_));
     prof_mark("embed");
     int ir = 0;
     for (const NvxRun &r : M.runs) {
         const NvxLayer &L = M.layers[(size_t)r.layer];
-        if (r.pass >= 0) {
+        if (r.pass > 0 && M.loop_add_embed) NVX_TRY(launch_add(x_, nvx_x0_, x_, (int64_t)T * W, stream_));   // a later pass opens with x += embedding rows
+        if (r.pass >= 0 && M.loop_in.w) {
             // x <- W_in [x ; x0] + step[pass]: the stream and the embedding output side by side, then the pass's own vector
             NVX_TRY(hipMemcpy2DAsync(nvx_xcat_, (size_t)2 * W * 4, x_, (size_t)W * 4, (size_t)W * 4, (size_t)T, hipMemcpyDeviceToDevice, stream_));
             NVX_TRY(nvx_linear(M.loop_in, nvx_xcat_, 2 * W, T, x_, W));
@@ -574,10 +580,12 @@ hipError_t Context::run_layers_novorax(int T) {
             NVX_TRY(nvx_linear(L.o, nvx_att_, H * L.vdim, T, nvx_y_, W));
             prof_mark("mlstm");
         } else if (L.type == NVX_GQ) {
-            NVX_TRY(nvx_linear(L.proj, x_, W, T, nvx_a_, L.proj.N, MMB_STORE, nullptr, 1.0f, L.norm1));
+            NVX_TRY(nvx_linear(L.proj, x_, W, T, nvx_a_, L.proj.N, MMB_STORE, nullptr, 1.0f, L.norm1, L.proj_bias));
             NVX_TRY(nvx_gq_attention(L, r, T));
         } else if (L.type == NVX_DELTA) {
             NVX_TRY(nvx_delta_mixer(L, r, T));
+        } else if (L.type == NVX_RETENTION) {
+            NVX_TRY(nvx_retention_mixer(L, r, T));
         } else return hipErrorInvalidValue;
         // norm on the sublayer's output, added to the stream (norm1 / norm2 in front of a sublayer are nullptr in a design whose sublayers read the stream itself)
         NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm1b, 1.0f, x_, x_, W, W, T, eps, stream_));

@@ -1,4 +1,4 @@
-// novorax.h — the layer stack of the folder models (config.json + model.safetensors, bf16 weights) as this runtime holds it.  Three designs fill it.
+// novorax.h — the layer stack of the folder models (config.json + model.safetensors, bf16 weights) as this runtime holds it.  Four designs fill it.
 //
 // Novorax: a decoder whose layers each pick a token mixer (latent attention with a sliding window and a
 // softmax sink, or the mLSTM matrix-memory recurrence) and a feed-forward (dense relu^2, or experts chosen by a token-id table), norms on both sides of every
@@ -20,6 +20,15 @@
 // sink; or the gated delta rule (short causal convolutions + silu on q / k / v, unit keys and queries, a write strength beta, a decay per head - "delta" - or per
 // head and key channel through a low-rank projection - "channel_delta" -, per-head unit-RMS output with a silu or a low-rank sigmoid gate).  Feed-forward:
 // W_down (gelu_tanh(W_gate x) * (W_up x)), or none.  The embedding rows enter times a constant and the same table is the output head.
+//
+// Dinilorn: norms on both sides of every sublayer (zero-centred weights).  Mixers: retention (linear attention with one fixed decay per head, rotate-half
+// rotary positions on q / k, keys over sqrt(dim), per-head unit-RMS output times silu(gate)); attention over every earlier token with projection biases, a
+// query multiplier that grows with the logarithm of the position, a soft cap, a learned bias per (distance bucket, head), one more term of score 0 in the softmax
+// denominator and a sigmoid gate per head; two-map attention (two score maps per head over the same values, neighbour-pair rotary positions with
+// three-band frequency scaling, a sliding window that keeps the first positions, a1 - lambda a2 normed per head, a sigmoid gate per entry).  Feed-forward:
+// experts g sigmoid(1.702 g) (u + 1) with clamped g, u; router = sigmoid scores, a selection bias that picks but does not weigh, expert groups scored by their two
+// best, un-normalised weights; a shared expert behind a one-number sigmoid gate.  A span of layers may run several times with shared weights; every pass but
+// the first opens with the embedding rows added to the stream.
 #pragma once
 
 #include <cstdint>
@@ -33,7 +42,8 @@ struct BfMat {                      // bf16 rows on the device
     int N = 0, K = 0;               // rows (outputs), row length (inputs)
 };
 
-enum { NVX_LATENT = 0, NVX_MLSTM = 1, NVX_GQ = 2, NVX_DELTA = 3 };   // token mixers: latent attention, matrix-memory recurrence, grouped-query attention, gated delta rule
+enum { NVX_LATENT = 0, NVX_MLSTM = 1, NVX_GQ = 2, NVX_DELTA = 3, NVX_RETENTION = 4 };   // token mixers: latent attention, matrix-memory recurrence, grouped-query attention, gated delta rule, retention
+enum { NVX_ROUTE_SOFTMAX_GROUPS = 0, NVX_ROUTE_SIGMOID_BIAS = 1 };   // routers of NVX_FF_ROUTED: softmax scores, groups by their best, normalised weights | sigmoid scores + selection bias, groups by their two best, raw weights
 enum { NVX_FF_NONE = 0, NVX_FF_DENSE = 1, NVX_FF_EXPERTS = 2, NVX_FF_ROUTED = 3 };   // dense; experts by a token-id table; experts by a router
 
 struct NvxLayer {
@@ -79,7 +89,26 @@ struct NvxLayer {
     int n_group = 1, group_keep = 1, shared_ff = 0;
     float router_scale = 1.0f;
     BfMat s_up, s_down;
-    int cache_row() const { return type == NVX_LATENT ? kv_rank + rot : type == NVX_GQ ? kv_heads * (dim + vdim) : 0; }   // f32 per cell of a run's cache plane
+    // ... with another router (route_kind; route_bias [n_expert] joins the scores for the choice only), gated experts (e_gate set: g sigmoid(1.702 g) (u + 1),
+    // g, u clamped by expert_limit; s_gate / shared_limit for the shared expert), and for a feed-forward that reads its own norm: route = [router ; shared gate]
+    // rows as a projection of its own (off_sg: the column of the shared expert's one-number sigmoid gate, -1: none)
+    int route_kind = NVX_ROUTE_SOFTMAX_GROUPS, off_sg = -1;
+    float *route_bias = nullptr;
+    float expert_limit = 0.0f, shared_limit = 0.0f;
+    BfMat route, s_gate;
+    // grouped-query attention, further switches: biases of the fused projection (zeros under the gate rows) and of W_o; a query multiplier
+    // 1 + q_temp_coef ln(floor((p + 1) / q_temp_every) + 1) (every 0: none); rel [rel_rows][heads] added to the score by distance bucket (dist_bucket [n_dist],
+    // longer distances take the last row); the first keep_first positions stay seen outside the window; rotary pairs (2i, 2i + 1); maps = 2: two score maps
+    // per head ([head][map][dim] rows of q and k) joined as unit_rms(a1 - map_lambda a2) * map_mult; the gate holds one number per output entry
+    float *proj_bias = nullptr, *o_bias = nullptr;
+    float q_temp_coef = 0.0f; int q_temp_every = 0;
+    float *rel = nullptr; int32_t *dist_bucket = nullptr; int n_dist = 0, rel_rows = 0;
+    int keep_first = 0, maps = 1;
+    bool rot_neighbours = false, gate_per_entry = false;
+    float map_lambda = 0.0f, map_mult = 1.0f;
+    // retention: proj = [q: heads*dim ; k: heads*dim ; v: heads*vdim ; g: heads*vdim] rows (off_g: the gate's column), decay [heads]; rot_dims / rot_freq as above
+    float *decay = nullptr;
+    int cache_row() const { return type == NVX_LATENT ? kv_rank + rot : type == NVX_GQ ? kv_heads * (maps * dim + vdim) : 0; }   // f32 per cell of a run's cache plane
 };
 
 struct NvxRun {
@@ -95,7 +124,9 @@ struct NovoraxModel {
     float *loop_step = nullptr;     // [times][width]
     float *final_norm = nullptr;
     float logit_scale = 1.0f, eps = 1e-5f, embed_scale = 1.0f;
-    std::string design;             // "novorax" | "fidepel" | "tuterax"
+    std::string design;             // "novorax" | "fidepel" | "tuterax" | "dinilorn"
+    bool loop_add_embed = false;    // every pass of the looped span but the first opens with x += embedding rows
+    int max_keep_first = 0;         // most first positions a windowed layer keeps seen (scan bounds)
     // norm weights: the factor is norm_off + w (1: zero-centred weights, 0: plain ones).  parallel_block: one norm per layer, mixer and feed-forward both read
     // it, x += residual_mult * (their sum); otherwise norms on both sides of each sublayer
     float norm_off = 1.0f, residual_mult = 1.0f;

@@ -182,13 +182,15 @@ class Context {
     hipError_t run_layers_novorax(int T);
     hipError_t run_output_novorax(int n_out, int out_base);
     hipError_t nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi = MMB_STORE, const BfMat *w2 = nullptr, float out_scale = 1.0f,
-                          const float *pn = nullptr);
+                          const float *pn = nullptr, const float *bias = nullptr, float epi_limit = 0.0f);
     hipError_t nvx_feed_forward(const NvxLayer &L, int T);
+    hipError_t nvx_routed_feed_forward(const NvxLayer &L, int T);            // dinilorn.cc: norm, [router ; shared gate] projection, routed + shared experts, weighted sum -> nvx_y_
+    hipError_t nvx_retention_mixer(const NvxLayer &L, const NvxRun &r, int T);   // dinilorn.cc: projection, recurrence, gated unit-RMS output, W_o -> nvx_y_
     // fidepel.cc: a block whose mixer and feed-forward read one norm; grouped-query attention on the run's cache plane; experts picked by a router
     hipError_t nvx_parallel_block(const NvxLayer &L, const NvxRun &r, int T);
     hipError_t nvx_gq_attention(const NvxLayer &L, const NvxRun &r, int T);
     hipError_t nvx_delta_mixer(const NvxLayer &L, const NvxRun &r, int T);   // tuterax.cc: projections, convolution, recurrence, gated unit-RMS output, W_o -> nvx_y_
-    hipError_t nvx_routed_experts(const NvxLayer &L, const float *h, const float *pn, int T);
+    hipError_t nvx_routed_experts(const NvxLayer &L, const float *h, const float *pn, int T, const float *z, int ld_z);   // z: the router's logits [T][n_expert], row stride ld_z
     hipError_t nvx_shared_expert(const NvxLayer &L, const float *h, const float *pn, int T);
     float *nvx_sh_ = nullptr, *nvx_ys_ = nullptr, *nvx_rw_ = nullptr;   // shared expert's hidden rows and output; router weights [T][top]
     // the three readers of a one-norm block's projection - attention, routed experts, shared expert - are independent until the block's closing sum: the two
