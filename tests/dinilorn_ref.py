@@ -107,7 +107,8 @@ def retention_scan(q, k, v, decay):
     return torch.stack(out)
 
 
-def retention(h, W, p, mx, eps):
+def retention(h, W, p, mx, eps, without=()):
+    """`without`: "state" (every token sees only itself)."""
     T = h.shape[0]
     H, D, VD = mx["heads"], mx["dim"], mx["vdim"]
     rot = mx.get("rot") or {}
@@ -116,7 +117,8 @@ def retention(h, W, p, mx, eps):
     q = turn_halves(lin(h, W, p + "q").reshape(T, H, D), pos, freq)
     k = turn_halves(lin(h, W, p + "k").reshape(T, H, D), pos, freq) * D ** -0.5
     v = lin(h, W, p + "v").reshape(T, H, VD)
-    o = rms_unit(retention_scan(q, k, v, torch.tensor(mx["decay"], dtype=F64)), eps).reshape(T, H * VD)
+    decay = torch.tensor(mx["decay"], dtype=F64) * (0.0 if "state" in without else 1.0)
+    o = rms_unit(retention_scan(q, k, v, decay), eps).reshape(T, H * VD)
     g = lin(h, W, p + "g")
     return lin(o * g * torch.sigmoid(g), W, p + "o")
 
@@ -180,7 +182,8 @@ def window_with_first(T, size, keep_first):
     return (dist >= 0) & ((dist < size) | (pos[None, :] < keep_first))
 
 
-def attention_two_maps(h, W, p, mx, eps, seen=None):
+def attention_two_maps(h, W, p, mx, eps, without=()):
+    """`without`: "keep_first" (the first positions are lost like any other), "window_wider" (one more position seen), "second_map" (lambda = 0)."""
     T = h.shape[0]
     H, G, D, VD = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
     pos = torch.arange(T)
@@ -189,11 +192,15 @@ def attention_two_maps(h, W, p, mx, eps, seen=None):
     q = turn_neighbours(lin(h, W, p + "q", True).reshape(T, H * 2, D), pos, freq).reshape(T, H, 2, D)
     k = turn_neighbours(lin(h, W, p + "k", True).reshape(T, G * 2, D), pos, freq).reshape(T, G, 2, D)
     v = lin(h, W, p + "v", True).reshape(T, G, VD)
-    if seen is None:
-        mask = mx.get("mask") or {}
-        seen = window_with_first(T, int(mask["size"]), int(mask.get("keep_first", 0))) if mask.get("size") else window_with_first(T, T + 1, 0)
+    mask = mx.get("mask") or {}
+    if mask.get("size"):
+        seen = window_with_first(T, int(mask["size"]) + (1 if "window_wider" in without else 0), 0 if "keep_first" in without else int(mask.get("keep_first", 0)))
+    else:
+        seen = window_with_first(T, T + 1, 0)
     diff = float(mx["diff"])
     lam = math.exp(float((W[p + "lq1"].to(F64) * W[p + "lk1"].to(F64)).sum())) - math.exp(float((W[p + "lq2"].to(F64) * W[p + "lk2"].to(F64)).sum())) + diff
+    if "second_map" in without:
+        lam = 0.0
     heads = []
     for a in range(H):
         g = a // (H // G)
@@ -229,16 +236,19 @@ def route(z, correction, top, groups, keep):
     return ids, s.gather(1, ids)
 
 
-def experts(h, W, p, mlp):
+def experts(h, W, p, mlp, without=()):
     rt = mlp["router"]
     gr = rt.get("groups") or {"count": 1, "keep": 1}
-    ids, w = route(lin(h, W, p + "router"), W[p + "correction"], rt["top"], gr["count"], gr["keep"])
+    if "groups" in without:
+        gr = {"count": 1, "keep": 1}
+    corr = W[p + "correction"] * (0.0 if "correction" in without else 1.0)
+    ids, w = route(lin(h, W, p + "router"), corr, rt["top"], gr["count"], gr["keep"])
     out = torch.zeros(h.shape[0], W[p + "e0.down"].shape[0], dtype=F64)
     for t in range(h.shape[0]):
         for j in range(ids.shape[1]):
             out[t] += w[t, j] * expert(h[t:t + 1], W, p + "e%d." % int(ids[t, j]), float(mlp["expert"]["limit"]))[0]
     sh = mlp.get("shared")
-    if sh:
+    if sh and "shared" not in without:
         out = out + torch.sigmoid(lin(h, W, p + "shared.sg")) * expert(h, W, p + "shared.", float(sh["limit"]))
     return out
 
@@ -256,28 +266,29 @@ def layer_runs(cfg):
     return runs + [(i, False) for i in range(b, n)]
 
 
-def forward(cfg, W, tokens, taps=None):
-    """logits [T, vocab] of one sequence; taps (a list) receives the stream after every layer run."""
+def forward(cfg, W, tokens, taps=None, without=()):
+    """logits [T, vocab] of one sequence; taps (a list) receives the stream after every layer run; `without` bends mechanisms (see the mixers; "reopen": the
+    passes of the looped span do not take the embedding rows in again; "correction": the router picks by its scores alone; "groups": every group stays open)."""
     eps = float(cfg["norm"]["eps"])
     x0 = W["embed"].to(F64)[torch.as_tensor(tokens, dtype=torch.long)]
     x = x0.clone()
     for il, reopen in layer_runs(cfg):
         lc = cfg["layers"][il]
         p = "l%d." % il
-        if reopen:
+        if reopen and "reopen" not in without:
             x = x + x0
         h = norm(x, W[p + "norm1"], eps)
         if lc["type"] == "retention":
-            y = retention(h, W, p + "mix.", lc["mixer"], eps)
+            y = retention(h, W, p + "mix.", lc["mixer"], eps, without)
         elif lc["type"] == "attention":
-            y = attention(h, W, p + "mix.", lc["mixer"])
+            y = attention(h, W, p + "mix.", lc["mixer"], without)
         elif lc["type"] == "attention_2":
-            y = attention_two_maps(h, W, p + "mix.", lc["mixer"], eps)
+            y = attention_two_maps(h, W, p + "mix.", lc["mixer"], eps, without)
         else:
             raise ValueError(lc["type"])
         x = x + norm(y, W[p + "norm1b"], eps)
         if lc.get("mlp"):
-            x = x + norm(experts(norm(x, W[p + "norm2"], eps), W, p + "mlp.", lc["mlp"]), W[p + "norm2b"], eps)
+            x = x + norm(experts(norm(x, W[p + "norm2"], eps), W, p + "mlp.", lc["mlp"], without), W[p + "norm2b"], eps)
         if taps is not None:
             taps.append(x.clone())
     return lin(norm(x, W["final.norm"], eps), W, "head")

@@ -1,0 +1,680 @@
+"""Dinilorn on the GPU against the float64 restatement in tests/dinilorn_ref.py (which processes whole sequences, with no cache, no state and no
+batching): every mechanism alone, prompts against token-by-token decoding, portions down to two tokens, mixed batches, cells and state slots that are
+used again, keys made loud on purpose (far back, at the window's edge, among the first positions a window keeps, at the causal edge), a memory that must
+hold for hundreds of tokens, first tokens, long decoding, odd sizes, the serving precision, graph replays, the engine's scheduler and the trace replay tool.
+
+The error of a logits row is the root mean square of (got - want) with the mean taken off, over the row's own root mean square.  Rows computed with
+exact_f32 differ from the float64 restatement by f32 rounding only: nine in ten rows stay within F32_TOL, every row within F32_WORST.  A wrong mechanism -
+a lost state, a key one position off, a bias row off by one - moves rows by 1e-3 and more; the tests that aim at one show that first."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import dinilorn_ref as R
+import dinilorn_synth as S
+
+pytestmark = pytest.mark.gpu
+F32_TOL = 2e-5
+F32_WORST = 3e-4
+BF16_TOL = 6e-2
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def row_errs(got, want):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    w = want - want.mean(-1, keepdims=True)
+    return np.sqrt((d ** 2).mean(-1)) / np.sqrt((w ** 2).mean(-1))
+
+
+def row_err(got, want):
+    return float(row_errs(got, want).max())
+
+
+def close(got, want):
+    e = row_errs(got, want)
+    return bool(e.max() <= F32_WORST and (len(e) < 10 or np.percentile(e, 90) <= F32_TOL))
+
+
+def toks(n, vocab, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+class Rig:
+    """A model folder, its weights for the oracle, and contexts of the product on it."""
+
+    def __init__(self, pkg, folder, cfg, seed=0, tweak=None):
+        self.cfg, self.W = cfg, S.weights(cfg, seed)
+        if tweak:
+            tweak(self.W)
+        self.dir = S.write(folder, cfg, self.W)
+        self.pkg = pkg
+        self.model = pkg.Model(self.dir)
+
+    def ctx(self, n_ctx=256, n_seq_max=4, exact=True, n_ubatch=64, graphs=True):
+        return self.pkg.Context(self.model, n_ctx=n_ctx, n_batch=max(n_ctx, n_ubatch), n_ubatch=n_ubatch, n_seq_max=n_seq_max, exact_f32=exact, use_graphs=graphs)
+
+    def ref(self, tokens, layers=False, without=()):
+        taps = [] if layers else None
+        out = R.forward(self.cfg, self.W, tokens, taps, without).numpy()
+        return (out, np.stack([t.numpy() for t in taps])) if layers else out
+
+
+def feed(ctx, tokens, start=0, seq=0, want_all=True):
+    """One decode call for tokens[start:] of a sequence; returns the logits of every fed position."""
+    n = len(tokens)
+    assert ctx.decode(tokens, list(range(start, start + n)), seq=[seq] * n, logits=[1] * n if want_all else None) == 0
+    return np.stack([ctx.logits(i) for i in range(n)]) if want_all else ctx.logits(-1)[None]
+
+
+def feed_in_portions(ctx, tokens, sizes, seq=0, start=0):
+    out, at, k = [], start, 0
+    while at < len(tokens):
+        n = min(sizes[k % len(sizes)], len(tokens) - at)
+        out.append(feed(ctx, tokens[at:at + n], at, seq))
+        at += n
+        k += 1
+    return np.concatenate(out)
+
+
+def one_by_one(ctx, tokens, start=0, seq=0):
+    return np.concatenate([feed(ctx, [tokens[i]], i, seq) for i in range(start, len(tokens))])
+
+
+FULL = [S.retention(mlp=S.moe()),
+        S.attention(mlp=S.moe(experts=8, top=3, groups=(2, 1), ff=16, shared=None)),
+        S.attention_2(mlp=S.moe(experts=5, top=1, groups=None)),
+        S.retention(heads=2, dim=8, vdim=40, rot_dims=0, mlp=None),
+        S.attention(heads=4, kv_heads=4, dim=12, vdim=12, softcap=0, q_temp=None, rel_rows=5, bias_max=9, mlp=None),
+        S.attention_2(heads=3, kv_heads=1, dim=16, vdim=8, rot_dims=16, scaling=None, size=0, mlp=S.moe(experts=4, top=2, groups=(4, 2), shared=(24, 0.8)))]
+
+
+@pytest.fixture(scope="module")
+def full(pkg, tmp_path_factory):
+    """Every branch in one small model: retention with and without turning entries, both attentions with shared and with own key heads, with and without a
+    window / cap / query multiplier, routers with and without groups, with groups of one, top 1 - 3, layers with and without a feed-forward or a shared
+    expert, and a looped span of three layers that runs twice."""
+    return Rig(pkg, tmp_path_factory.mktemp("dnl_full"), S.config(FULL, loop=(1, 4, 2)), seed=3)
+
+
+# ------------------------------------------------------------------------------------------ each mechanism alone
+@pytest.mark.parametrize("name,layers,loop", [
+    ("retention", [S.retention()], None),
+    ("retention_whole_head_turns", [S.retention(heads=2, dim=12, vdim=20, rot_dims=12)], None),
+    ("retention_nothing_turns", [S.retention(rot_dims=0, decay=[0.5, 0.99, 1.0])], None),
+    ("retention_wide_values", [S.retention(heads=2, dim=24, vdim=136)], None),
+    ("attention", [S.attention()], None),
+    ("attention_every_head_its_own_key", [S.attention(heads=3, kv_heads=3)], None),
+    ("attention_no_cap_no_multiplier", [S.attention(softcap=0, q_temp=None, scale=0.5)], None),
+    ("attention_two_bias_rows", [S.attention(rel_rows=2, bias_max=3)], None),
+    ("attention_odd_bias_rows", [S.attention(rel_rows=7, bias_max=11)], None),
+    ("attention_2", [S.attention_2()], None),
+    ("attention_2_every_head_its_own_key", [S.attention_2(heads=2, kv_heads=2)], None),
+    ("attention_2_whole_head_turns_no_window", [S.attention_2(rot_dims=12, size=0)], None),
+    ("attention_2_plain_frequencies", [S.attention_2(scaling=None, keep_first=0, size=4)], None),
+    ("attention_2_nothing_turns", [S.attention_2(rot_dims=0, size=1, keep_first=2)], None),
+    ("experts", [S.retention(heads=1, dim=8, vdim=8, rot_dims=2, mlp=S.moe())], None),
+    ("experts_no_groups_top_one", [S.retention(heads=1, dim=8, vdim=8, rot_dims=2, mlp=S.moe(experts=5, top=1, groups=None))], None),
+    ("experts_every_group_kept", [S.retention(heads=1, dim=8, vdim=8, rot_dims=2, mlp=S.moe(experts=6, top=4, groups=(2, 2)))], None),
+    ("experts_groups_of_one_no_shared", [S.retention(heads=1, dim=8, vdim=8, rot_dims=2, mlp=S.moe(experts=4, top=2, groups=(4, 3), shared=None))], None),
+    ("looped_span", [S.retention(mlp=S.moe()), S.attention(), S.attention_2(mlp=S.moe(top=1))], (0, 2, 3)),
+    ("whole_model_looped", [S.attention_2(), S.retention(mlp=S.moe())], (0, 2, 2)),
+])
+def test_mechanism_alone_matches_the_restatement(pkg, tmp_path, name, layers, loop):
+    rig = Rig(pkg, tmp_path / name, S.config(layers, loop=loop), seed=11)
+    t = toks(29, rig.cfg["vocab"], 5)
+    want, taps = rig.ref(t, layers=True)
+    c = rig.ctx()
+    c.enable_taps(True)
+    got = feed(c, t)
+    for r in range(taps.shape[0]):
+        assert np.abs(c.layer_out(r, len(t)) - taps[r]).max() <= 1e-4 * max(1.0, np.abs(taps[r]).max()), (name, r)
+    assert close(got, want)
+    assert close(one_by_one(rig.ctx(), t), want)
+
+
+def test_the_restatement_tells_the_parts_apart(pkg, tmp_path):
+    """Each part moves the logits of this model by far more than the tolerance: the product can only agree with the restatement if it has every one."""
+    cfg = S.config([S.retention(mlp=S.moe(experts=8, top=2, groups=(4, 2))), S.attention(scale=0.6, softcap=3.0), S.attention_2(size=5, keep_first=2)], loop=(0, 3, 2))
+    rig = Rig(pkg, tmp_path / "parts", cfg, seed=12)
+    t = toks(40, rig.cfg["vocab"], 6)
+    want = rig.ref(t)
+    for part in ("sink", "bias", "softcap", "temperature", "gate", "keep_first", "window_wider", "second_map", "state", "reopen", "correction", "groups", "shared"):
+        assert row_err(rig.ref(t, without=(part,)), want) > 1e-2, part
+    assert close(feed(rig.ctx(), t), want)
+    assert close(feed_in_portions(rig.ctx(), t, [7, 2, 1, 11]), want)
+
+
+def test_the_router_alone(pkg, tmp_path):
+    """Twelve experts in four groups with selection biases from -3 to 2: choice scores that are negative, best experts inside closed groups, groups that win
+    by their second best.  The stream behind the feed-forward and the logits agree with the restatement; the restatement without the bias, or with every
+    group open, does not."""
+    E, top = 12, 3
+    mlp = S.moe(experts=E, top=top, groups=(4, 2), ff=8, shared=None)
+    rig = Rig(pkg, tmp_path / "router", S.config([S.retention(heads=1, dim=8, vdim=8, rot_dims=0, mlp=mlp)], width=48, vocab=200), seed=21,
+              tweak=lambda W: W.__setitem__("l0.mlp.correction", torch.tensor([-3.0, 0.4, -0.2, 0.9, 0.0, -1.5, 0.3, 0.3, 2.0, -2.0, -2.0, 0.1]).to(torch.bfloat16)))
+    t = toks(120, 200, 3)
+    want, taps = rig.ref(t, layers=True)
+    c = rig.ctx(n_ubatch=128)
+    c.enable_taps(True)
+    got = feed(c, t, want_all=True)
+    assert np.abs(c.layer_out(0, len(t)) - taps[0]).max() <= 1e-4 * np.abs(taps[0]).max()
+    assert close(got, want)
+    for part in ("correction", "groups"):
+        assert row_err(rig.ref(t, without=(part,)), want) > 1e-2, part
+
+
+# ------------------------------------------------------------------------------------------ prompts, single tokens, portions
+def test_prompt_equals_token_by_token(full):
+    t = toks(45, full.cfg["vocab"], 1)
+    want = full.ref(t)
+    whole = feed(full.ctx(), t)
+    single = one_by_one(full.ctx(), t)
+    assert close(whole, want) and close(single, want)
+    assert close(single, whole)
+
+
+@pytest.mark.parametrize("sizes", [[2], [3, 2, 7], [17, 2, 2, 30], [64, 5], [1, 2, 1, 9], [12, 11, 13], [31, 1, 32, 33], [1, 1, 2, 1, 3]])
+def test_portions_of_any_size(full, sizes):
+    """Portions that end on and beside the recurrence kernel's staging chunks and reduction rounds (8 and 32 tokens), that cut the 9-token window and the
+    three kept positions, and portions above 32 that the engine cuts again."""
+    t = toks(97, full.cfg["vocab"], 2)
+    got = feed_in_portions(full.ctx(n_ubatch=32), t, sizes)
+    assert close(got, full.ref(t))
+
+
+def test_long_decoding_after_a_prompt(full):
+    t = toks(300, full.cfg["vocab"], 4)
+    c = full.ctx(n_ctx=320)
+    got = np.concatenate([feed(c, t[:40]), one_by_one(c, t, 40)])
+    assert close(got, full.ref(t))
+
+
+def test_the_first_tokens_of_a_sequence(full):
+    """Position 0 sees one key (and the term of score 0), the memory is empty, the window and the kept positions coincide."""
+    t = toks(4, full.cfg["vocab"], 9)
+    want = full.ref(t)
+    assert close(feed(full.ctx(), t), want)
+    assert close(one_by_one(full.ctx(), t), want)
+    assert close(feed_in_portions(full.ctx(), t, [1, 3]), want)
+    assert close(feed(full.ctx(), t[:1]), want[:1])
+
+
+# ------------------------------------------------------------------------------------------ batches, cells and slots used again
+def test_unequal_requests_in_one_batch_equal_each_alone(full):
+    V = full.cfg["vocab"]
+    reqs = [toks(n, V, 120 + i) for i, n in enumerate((37, 9, 61, 1))]
+    want = [full.ref(r) for r in reqs]
+    c = full.ctx(n_ctx=192, n_ubatch=48)                     # (48 cells per sequence region: the 61-token request spills into its neighbours')
+    at = [0] * len(reqs)
+    got = [[] for _ in reqs]
+    plan = [(5, 1, 30, 1), (2, 1, 2, 0), (1, 1, 29, 0), (29, 6, 0, 0), (0, 0, 0, 0)]
+    while any(at[i] < len(reqs[i]) for i in range(len(reqs))):
+        for step in plan:
+            tk, ps, sq, owner = [], [], [], []
+            for i, n in enumerate(step):
+                n = min(n if n else 1, len(reqs[i]) - at[i])
+                tk += reqs[i][at[i]:at[i] + n]; ps += list(range(at[i], at[i] + n)); sq += [i] * n; owner += [i] * n
+                at[i] += n
+            if not tk:
+                continue
+            assert c.decode(tk, ps, seq=sq, logits=[1] * len(tk)) == 0
+            for j, i in enumerate(owner):
+                got[i].append(c.logits(j))
+    for i in range(len(reqs)):
+        assert close(np.stack(got[i]), want[i]), i
+
+
+def test_a_sequence_that_comes_back_later_in_the_batch(full):
+    """Rows of one sequence in two runs of the same batch, another sequence between them: the second run must start from the state the first one left."""
+    V = full.cfg["vocab"]
+    a, b = toks(20, V, 83), toks(6, V, 81)
+    c = full.ctx()
+    tk = a[:7] + b + a[7:20]
+    ps = list(range(7)) + list(range(6)) + list(range(7, 20))
+    sq = [0] * 7 + [1] * 6 + [0] * 13
+    assert c.decode(tk, ps, seq=sq, logits=[1] * len(tk)) == 0
+    got = np.stack([c.logits(i) for i in range(len(tk))])
+    assert close(np.concatenate([got[:7], got[13:]]), full.ref(a))
+    assert close(got[7:13], full.ref(b))
+
+
+def test_cells_and_state_slots_are_used_again(full):
+    """A context with room for one request at a time: every request takes the cells and the slot its predecessor gave back - a memory that kept anything
+    of the predecessor would show at once; then two live requests, one ends and a third takes its slot beside the survivor."""
+    V = full.cfg["vocab"]
+    c = full.ctx(n_ctx=64, n_seq_max=2)
+    for k in range(5):
+        t = toks(50 + k, V, 40 + k)
+        got = feed_in_portions(c, t, [13, 2, 21], seq=k % 2)
+        assert close(got, full.ref(t)), k
+        assert c.kv_used() == len(t)
+        assert c.kv_seq_rm(k % 2, -1, -1)
+        assert c.kv_used() == 0
+    a, b, d = toks(30, V, 50), toks(34, V, 51), toks(28, V, 52)
+    ga = feed(c, a, 0, 0)
+    gb = feed(c, b[:20], 0, 1)
+    assert c.kv_seq_rm(0, -1, -1)
+    gd = feed(c, d, 0, 0)
+    gb = np.concatenate([gb, feed(c, b[20:], 20, 1)])
+    for got, t in ((ga, a), (gb, b), (gd, d)):
+        assert close(got, full.ref(t))
+
+
+def test_a_recurrent_sequence_cannot_be_cut_back_but_can_be_copied(full):
+    t = toks(40, full.cfg["vocab"], 7)
+    c = full.ctx()
+    feed(c, t[:25])
+    assert not c.kv_seq_rm(0, 12, -1)                           # the state has absorbed positions 12 .. 24
+    c.kv_seq_cp(0, 2, 0, -1)                                    # cells and state of the whole sequence
+    tail = toks(15, full.cfg["vocab"], 8)
+    got0 = feed(c, t[25:], 25, 0)
+    got2 = feed(c, tail, 25, 2)
+    assert close(got0, full.ref(t)[25:])
+    assert close(got2, full.ref(t[:25] + tail)[25:])
+
+
+# ------------------------------------------------------------------------------------------ keys and memories made loud
+D0 = 12                                                         # the loud coordinate: beyond the turning entries of the two-map layer below
+
+
+def _loud_rig(pkg, folder, layer, gain=4.0, seed=4):
+    """One attention layer with a nearly one-hot softmax: coordinate D0 of the first query head (first map) and of its key head is made loud through the
+    rows of the two projections, so the score is decided by that coordinate."""
+    def tweak(W):
+        W["l0.mix.q"][D0] *= gain
+        W["l0.mix.k"][D0] *= gain
+    return Rig(pkg, folder, S.config([layer], width=48, vocab=50), seed=seed, tweak=tweak)
+
+
+def _loud_sequence(rig, n, p0, askers, seed=6):
+    """n tokens whose keys are quiet in the loud coordinate, except ONE token at position p0 whose key is the loudest of the vocabulary; the rows in `askers`
+    hold the quiet token whose query asks for it most.  A row that sees p0 gives it nearly all its weight (in the loud map)."""
+    F64, W, eps = torch.float64, rig.W, rig.cfg["norm"]["eps"]
+    h = R.norm(W["embed"].to(F64), W["l0.norm1"], eps)             # the mixer's input of a one-layer model is decided by the token alone
+    k = R.lin(h, W, "l0.mix.k", True)[:, D0]
+    q = R.lin(h, W, "l0.mix.q", True)[:, D0]
+    loud = int(torch.argmax(k))
+    quiet = [int(i) for i in torch.argsort(k.abs()) if int(i) != loud][:30]
+    asker = max(quiet, key=lambda i: float(q[i]))
+    t = [quiet[int(i)] for i in torch.randint(0, len(quiet), (n,), generator=torch.Generator().manual_seed(seed))]
+    t[p0] = loud
+    for r in askers:
+        t[r] = asker
+    return t, quiet
+
+
+LOUD_ATTENTION = S.attention(heads=2, kv_heads=1, dim=16, vdim=16, scale=1.0, softcap=60.0, rel_rows=12, bias_max=200)
+
+
+@pytest.mark.parametrize("p0,far", [(0, 300), (5, 250), (63, 129), (64, 448)])
+def test_a_far_key_among_hundreds(pkg, tmp_path, p0, far):
+    """One loud key hundreds of positions back, at the first cell, at a cell region's last and at the next region's first cell: the asking row far behind
+    gives it nearly all its weight (the restatement with another token in its place changes that row outright).  Whole prompts, portions cut by the
+    micro-batch, single tokens, and a prompt that ends just before the asking row."""
+    rig = _loud_rig(pkg, tmp_path / "loud", LOUD_ATTENTION)
+    r = p0 + far
+    n = r + 7
+    t, quiet = _loud_sequence(rig, n, p0, [r, r + 3])
+    want = rig.ref(t)
+    other = list(t)
+    other[p0] = quiet[0]
+    e = row_errs(rig.ref(other), want)
+    assert e[r] > 0.01 and e[r + 3] > 0.01                      # (of the logits row's own spread; the mixer's share of the stream bounds it)
+    n_ctx = (n + 63) // 64 * 64
+    assert close(feed(rig.ctx(n_ctx=n_ctx, n_ubatch=512), t), want)
+    assert close(feed_in_portions(rig.ctx(n_ctx=n_ctx, n_ubatch=128), t, [r, 2, 100]), want)    # the asking row opens a two-token portion
+    assert close(feed_in_portions(rig.ctx(n_ctx=n_ctx, n_ubatch=128), t, [r + 1, 100]), want)    # ... and closes a prompt portion
+    c = rig.ctx(n_ctx=n_ctx, n_ubatch=128)
+    got = np.concatenate([feed_in_portions(c, t[:r - 2], [128, 3, 100]), one_by_one(c, t, r - 2)])
+    assert close(got, want)
+
+
+def test_the_causal_edge(pkg, tmp_path):
+    """The loud key at position p0: the asking row at p0 + 1 sees it, the one at p0 - 1 must not - also when both are rows of the same batch."""
+    rig = _loud_rig(pkg, tmp_path / "edge", LOUD_ATTENTION)
+    for p0 in (1, 31, 32, 40):
+        t, quiet = _loud_sequence(rig, p0 + 12, p0, [p0 - 1, p0 + 1])
+        want = rig.ref(t)
+        other = list(t)
+        other[p0] = quiet[0]
+        e = row_errs(rig.ref(other), want)
+        assert e[p0 + 1] > 0.05 and e[p0 - 1] == 0.0, p0
+        assert close(feed(rig.ctx(), t), want)
+        assert close(feed_in_portions(rig.ctx(), t, [p0, 2, 5]), want)        # the key opens a portion
+        assert close(feed_in_portions(rig.ctx(), t, [p0 + 1, 2, 5]), want)    # ... and closes one
+        c = rig.ctx()
+        assert close(np.concatenate([feed(c, t[:max(p0 - 1, 1)]), one_by_one(c, t, max(p0 - 1, 1))]), want)
+
+
+def test_the_term_of_score_zero_takes_its_share_once(pkg, tmp_path):
+    """Scores far below zero in one head (a large negative bias row for every distance), ordinary ones in the other: the first head gives nearly all its
+    weight to the term that has no value, so the heads enter the output in another proportion than under a plain softmax.  Leaving the term out, or counting
+    it once per split of a scan, would change nearly every row."""
+    def tweak(W):
+        W["l0.mix.rel"][:, 0] = -9.0
+    rig = Rig(pkg, tmp_path / "sink", S.config([S.attention(heads=2, kv_heads=1, dim=16, vdim=16, rel_rows=6, bias_max=30)], width=48, vocab=50), seed=4, tweak=tweak)
+    t = toks(200, 50, 16)
+    want = rig.ref(t)
+    assert np.median(row_errs(rig.ref(t, without=("sink",)), want)) > 1e-2
+    assert close(feed(rig.ctx(n_ubatch=256), t), want)
+    c = rig.ctx()
+    assert close(np.concatenate([feed_in_portions(c, t[:150], [64]), one_by_one(c, t, 150)]), want)
+
+
+@pytest.mark.parametrize("size,keep", [(64, 3), (9, 0), (130, 17)])
+def test_the_window_edge_and_the_kept_first_positions(pkg, tmp_path, size, keep):
+    """Two-map attention, the loud key at p0 >= keep: the asking row at distance size - 1 gives it nearly all the first map's weight, the row at distance size
+    has lost it.  The loud key at position keep - 1 is seen from any distance, at position keep it is lost like any other.  Whole prompts, the asking rows
+    as first and as last row of a portion, single tokens across the edges."""
+    layer = S.attention_2(heads=2, kv_heads=1, dim=16, vdim=16, scale=1.0, rot_dims=8, size=size, keep_first=keep, diff=0.3)
+    rig = _loud_rig(pkg, tmp_path / "win", layer)
+    cases = [(keep + 21, "window_wider")]
+    if keep:
+        cases += [(keep - 1, "keep_first"), (keep, None)]
+    for p0, bent in cases:
+        r_in, r_out = p0 + size - 1, p0 + size
+        n = r_out + 40
+        far = r_out + 30
+        t, quiet = _loud_sequence(rig, n, p0, [r_in, r_out, far])
+        want = rig.ref(t)
+        other = list(t)
+        other[p0] = quiet[0]
+        e = row_errs(rig.ref(other), want)
+        assert e[r_in] > 0.05, (p0, e[r_in])
+        if bent == "keep_first":                                 # a kept position: the far row still sees it; the restatement that forgets the rule does not
+            assert e[far] > 0.05 and e[r_out] > 0.05
+            assert row_errs(rig.ref(t, without=("keep_first",)), want)[far] > 0.05
+        else:
+            assert e[r_out] == 0.0 and e[far] == 0.0
+            assert row_errs(rig.ref(t, without=("window_wider",)), want)[r_out] > 0.05
+        n_ctx = (n + 63) // 64 * 64
+        assert close(feed(rig.ctx(n_ctx=n_ctx, n_ubatch=512), t), want)
+        assert close(feed_in_portions(rig.ctx(n_ctx=n_ctx), t, [r_in, 2, 50]), want)         # r_in opens a two-token portion whose other row is r_out
+        assert close(feed_in_portions(rig.ctx(n_ctx=n_ctx), t, [r_out, 2, 50]), want)        # r_out opens one; r_in closed the prompt portion
+        c = rig.ctx(n_ctx=n_ctx)
+        start = max(r_in - 2, 1)
+        assert close(np.concatenate([feed_in_portions(c, t[:start], [64, 3]), one_by_one(c, t, start)]), want)
+
+
+def test_a_windowed_request_beside_requests_that_come_and_go(pkg, tmp_path):
+    """A long request decodes through its window while short requests beside it start, end and hand their cells and slots on."""
+    cfg = S.config([S.attention_2(size=20, keep_first=4, mlp=S.moe()), S.retention(), S.attention(mlp=S.moe(top=1, groups=None))], loop=(0, 2, 2))
+    rig = Rig(pkg, tmp_path / "beside", cfg, seed=8)
+    V = cfg["vocab"]
+    long_t = toks(150, V, 70)
+    c = rig.ctx(n_ctx=256, n_seq_max=3, n_ubatch=32)
+    got_long = [feed(c, long_t[:30], 0, 0)]
+    at, k = 30, 0
+    while at < len(long_t):
+        short = toks(5 + 3 * (k % 4), V, 200 + k)
+        slot = 1 + k % 2
+        tk = [long_t[at]] + short
+        ps = [at] + list(range(len(short)))
+        sq = [0] + [slot] * len(short)
+        assert c.decode(tk, ps, seq=sq, logits=[1] * len(tk)) == 0
+        rows = np.stack([c.logits(i) for i in range(len(tk))])
+        got_long.append(rows[:1])
+        assert close(rows[1:], rig.ref(short)), k
+        assert c.kv_seq_rm(slot, -1, -1)
+        at += 1
+        k += 1
+    assert close(np.concatenate(got_long), rig.ref(long_t))
+
+
+def test_a_memory_that_holds_hundreds_of_tokens(pkg, tmp_path):
+    """Decays close to one: what token 60 wrote is still read 240 and more tokens later (the restatement with another token there differs at those rows) -
+    through micro-batches, portions of two and single tokens."""
+    cfg = S.config([S.retention(heads=2, dim=24, vdim=16, rot_dims=8, decay=[0.9990234375, 0.99951171875])], width=48, vocab=50)
+    rig = Rig(pkg, tmp_path / "hold", cfg, seed=5)
+    t = toks(330, 50, 17)
+    want = rig.ref(t)
+    other = list(t)
+    other[60] = (t[60] + 1) % 50
+    assert row_errs(rig.ref(other), want)[300:].min() > 2e-3
+    assert close(feed(rig.ctx(n_ctx=384, n_ubatch=512), t), want)
+    assert close(feed_in_portions(rig.ctx(n_ctx=384, n_ubatch=48), t, [100, 2, 2, 150]), want)
+    c = rig.ctx(n_ctx=384)
+    assert close(np.concatenate([feed_in_portions(c, t[:290], [64]), one_by_one(c, t, 290)]), want)
+
+
+def test_distance_buckets_up_to_the_last_row(pkg, tmp_path):
+    """A bias table whose rows differ by whole units and a model that is otherwise nearly blind to position: rows at every distance up to beyond bias_max,
+    where the log-spaced buckets change and where they end."""
+    def tweak(W):
+        W["l0.mix.rel"][:] = (torch.arange(9, dtype=torch.float32)[:, None] * torch.tensor([1.0, -0.7])[None, :]).to(torch.bfloat16)
+    rig = Rig(pkg, tmp_path / "buckets", S.config([S.attention(heads=2, kv_heads=2, dim=8, vdim=8, scale=0.05, softcap=0, q_temp=None, rel_rows=9, bias_max=64)],
+                                                  width=40, vocab=30), seed=2, tweak=tweak)
+    t = toks(90, 30, 3)
+    want = rig.ref(t)
+    assert close(feed(rig.ctx(n_ubatch=128), t), want)
+    assert close(one_by_one(rig.ctx(), t), want)
+    assert row_err(rig.ref(t, without=("bias",)), want) > 1e-2
+
+
+# ------------------------------------------------------------------------------------------ other sizes
+@pytest.mark.parametrize("name,layers,width,vocab,loop", [
+    ("ones", [S.retention(heads=1, dim=2, vdim=1, rot_dims=2, decay=[0.9], mlp=S.moe(experts=1, top=1, groups=(1, 1), ff=1, shared=(1, 1.0))),
+              S.attention(heads=1, kv_heads=1, dim=1, vdim=1, rel_rows=2, bias_max=2, q_temp=(0.3, 1)),
+              S.attention_2(heads=1, kv_heads=1, dim=2, vdim=1, rot_dims=2, size=1, keep_first=1)], 24, 11, (1, 2, 1)),
+    ("retention_dim_144_vdim_200", [S.retention(heads=2, dim=144, vdim=200, rot_dims=64)], 64, 50, None),
+    ("retention_dim_300", [S.retention(heads=1, dim=300, vdim=72, rot_dims=300)], 64, 50, None),
+    ("retention_dim_40_unaligned", [S.retention(heads=5, dim=40, vdim=7, rot_dims=14)], 44, 50, None),
+    ("attention_dim_160_vdim_272", [S.attention(heads=2, kv_heads=1, dim=160, vdim=272, scale=0.1)], 64, 50, None),
+    ("attention_unaligned_heads", [S.attention(heads=4, kv_heads=2, dim=10, vdim=14), S.attention_2(heads=3, kv_heads=3, dim=10, vdim=7, rot_dims=6)], 50, 53, None),
+    ("attention_2_dim_320_vdim_256", [S.attention_2(heads=2, kv_heads=2, dim=320, vdim=256, rot_dims=128, scale=0.06, size=33, keep_first=5)], 64, 50, None),
+    ("attention_2_many_heads", [S.attention_2(heads=24, kv_heads=3, dim=8, vdim=8, rot_dims=4, size=6, keep_first=9)], 72, 50, None),
+    ("bias_table_far_reach", [S.attention(heads=3, kv_heads=1, dim=8, vdim=8, rel_rows=32, bias_max=5000)], 40, 50, None),
+    ("seventy_experts", [S.retention(heads=1, dim=8, vdim=8, mlp=S.moe(experts=70, top=3, groups=(7, 3), ff=8))], 40, 50, None),
+    ("wide_experts_width_50", [S.retention(heads=1, dim=8, vdim=8, mlp=S.moe(experts=3, top=2, groups=None, ff=130, shared=(70, 0.5)))], 50, 50, None),
+    ("span_at_the_end_four_passes", [S.attention(), S.retention(mlp=S.moe()), S.attention_2()], 72, 97, (1, 3, 4)),
+])
+def test_other_sizes(pkg, tmp_path, name, layers, width, vocab, loop):
+    rig = Rig(pkg, tmp_path / name, S.config(layers, width=width, vocab=vocab, loop=loop), seed=13)
+    t = toks(70, vocab, 14)
+    want = rig.ref(t)
+    assert close(feed(rig.ctx(n_ubatch=128), t), want), name
+    assert close(feed_in_portions(rig.ctx(), t, [33, 2, 1, 17]), want), name
+    c = rig.ctx()
+    assert close(np.concatenate([feed(c, t[:50]), one_by_one(c, t, 50)]), want), name
+
+
+def test_a_wide_vocabulary_with_few_rows(pkg, tmp_path):
+    rig = Rig(pkg, tmp_path / "vocab", S.config([S.retention(heads=1, dim=8, vdim=8)], width=64, vocab=4099), seed=15)
+    t = toks(9, 4099, 16)
+    want = rig.ref(t)
+    for n in (1, 2, 3, 4):
+        assert close(feed(rig.ctx(), t[:n]), want[:n]), n
+
+
+def _random_layer(rng):
+    pick = lambda xs: xs[int(rng.integers(len(xs)))]
+    mlp = None
+    if rng.random() < 0.6:
+        groups = pick([None, (2, 1), (3, 2), (2, 2)])
+        per = pick([2, 3, 4])
+        experts = per * (groups[0] if groups else pick([1, 2, 3]))
+        top = pick([t for t in (1, 2, 3) if t <= (per * groups[1] if groups else experts)])
+        mlp = S.moe(experts=experts, top=top, groups=groups, ff=pick([8, 24, 40]), limit=pick([0.7, 1.5]), shared=pick([None, (16, 1.0), (48, 2.0)]))
+    kind = pick(["retention", "attention", "attention_2"])
+    if kind == "retention":
+        heads, dim = pick([1, 2, 4]), pick([16, 32, 64])
+        return S.retention(heads=heads, dim=dim, vdim=pick([16, 48, 80]), rot_dims=pick([0, 8, dim]), mlp=mlp)
+    heads, share = pick([1, 2, 4, 8]), pick([1, 2, 4])
+    kv = max(heads // share, 1)
+    dim = pick([16, 32, 64])
+    if kind == "attention":
+        rows = pick([4, 9, 16])
+        return S.attention(heads=heads, kv_heads=kv, dim=dim, vdim=pick([16, 32, 64]), scale=dim ** -0.5, softcap=pick([0, 5.0, 30.0]), rel_rows=rows,
+                           bias_max=pick([rows, 40, 300]), q_temp=pick([None, (0.2, 7), (0.5, 64)]), mlp=mlp)
+    return S.attention_2(heads=heads, kv_heads=kv, dim=dim, vdim=pick([16, 32, 64]), scale=dim ** -0.5, rot_dims=pick([0, 8, dim]),
+                         scaling=pick([None, (8.0, 1.0, 4.0, 128), (2.0, 0.5, 2.0, 40)]), size=pick([0, 3, 50, 64, 100]), keep_first=pick([0, 1, 6]),
+                         diff=pick([0.2, 0.5, 0.8]), mlp=mlp)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_random_configurations(pkg, tmp_path, seed):
+    """Four to eight layers of any kind in any order with sizes drawn from lists, a looped span somewhere; a 400-token request in portions of changing size
+    and single tokens beside a short request that comes and goes."""
+    rng = np.random.default_rng(seed)
+    layers = [_random_layer(rng) for _ in range(int(rng.integers(4, 9)))]
+    a = int(rng.integers(0, len(layers)))
+    b = int(rng.integers(a + 1, len(layers) + 1))
+    cfg = S.config(layers, width=int(rng.choice([64, 88, 128])), vocab=int(rng.choice([101, 256])), loop=(a, b, int(rng.integers(1, 4))))
+    rig = Rig(pkg, tmp_path / f"random{seed}", cfg, seed=100 + seed)
+    V = cfg["vocab"]
+    long_t, short = toks(400, V, 7 + seed), toks(23, V, 9 + seed)
+    want_long, want_short = rig.ref(long_t), rig.ref(short)
+    c = rig.ctx(n_ctx=512, n_seq_max=2, n_ubatch=128)
+    got_long, got_short, at, sat = [], [], 0, 0
+    sizes = [150, 2, 1, 64, 1, 1, 37, 3, 1, 1, 1, 90, 1, 2]
+    k = 0
+    while at < len(long_t):
+        n = min(sizes[k % len(sizes)], len(long_t) - at)
+        m = min([5, 1, 1, 9, 2][k % 5], len(short) - sat)
+        tk = long_t[at:at + n] + short[sat:sat + m]
+        ps = list(range(at, at + n)) + list(range(sat, sat + m))
+        sq = [0] * n + [1] * m
+        assert c.decode(tk, ps, seq=sq, logits=[1] * len(tk)) == 0
+        rows = np.stack([c.logits(i) for i in range(len(tk))])
+        got_long.append(rows[:n])
+        got_short.append(rows[n:])
+        at += n
+        sat += m
+        if sat == len(short):                                   # the short request ends, gives its cells and slot back and starts over
+            assert close(np.concatenate(got_short), want_short), (seed, k)
+            assert c.kv_seq_rm(1, -1, -1)
+            got_short, sat = [], 0
+        k += 1
+    assert close(np.concatenate(got_long), want_long), seed
+
+
+# ------------------------------------------------------------------------------------------ precision, graphs
+def test_serving_precision(full):
+    """exact_f32 off: batches round their activations to bf16 for the matrix cores; positions, scores, softmax, norms, the router's arithmetic, the recurrence
+    and the stream stay f32.  Single tokens keep f32 activations."""
+    t = toks(96, full.cfg["vocab"], 30)
+    want = full.ref(t)
+    exact = feed(full.ctx(n_ubatch=128), t)
+    bf = feed(full.ctx(exact=False, n_ubatch=128), t)
+    e = row_errs(bf, want)
+    assert np.median(e) <= 2e-2 and np.percentile(e, 90) <= BF16_TOL, (np.median(e), np.percentile(e, 90), e.max())
+    assert row_err(bf, exact) > 1e-5                              # (activations were rounded to bf16: another kernel ran)
+    single = one_by_one(full.ctx(exact=False), t)
+    assert close(single, want)
+
+
+def test_graph_replays_equal_eager_steps(full):
+    t = toks(40, full.cfg["vocab"], 31)
+    outs = []
+    for graphs in (True, False):
+        c = full.ctx(graphs=graphs)
+        feed(c, t[:8], want_all=False)
+        rows = []
+        for i in range(8, len(t)):
+            rows.append(feed(c, [t[i]], i, want_all=False)[0])
+            if i % 7 == 0:
+                c.synchronize()
+        outs.append(np.stack(rows))
+    assert np.array_equal(outs[0], outs[1])
+    assert close(outs[0], full.ref(t)[8:])
+
+
+# ------------------------------------------------------------------------------------------ the engine and the tools
+def test_greedy_generation_through_the_engine(pkg, full):
+    """loadmodel -> chat completion through the slot scheduler, two requests side by side; the text is decimal token ids."""
+    V = full.cfg["vocab"]
+    e = pkg.Engine()
+    try:
+        st, body = e.load_model(llama_model_path=full.dir, model="dnl", ctx_len=256, n_parallel=2, ngl=100, exact_f32=True, user_prompt="", ai_prompt="", system_prompt="")
+        assert st["status_code"] == 200 and not st["has_error"], (st, body)
+        prompts = [toks(11, V, 60), toks(23, V, 61)]
+        n_new = 12
+
+        def greedy(p):
+            seq = list(p)
+            for _ in range(n_new + 1):
+                seq.append(int(np.argmax(full.ref(seq)[-1])))
+            return seq[len(p):]
+
+        import threading
+        out = [None, None]
+
+        def run(i):
+            res = e.chat_completion(model="dnl", messages=[{"role": "user", "content": " ".join(map(str, prompts[i]))}], max_tokens=n_new, temperature=0.0,
+                                    repeat_penalty=1.0, frequency_penalty=0.0, presence_penalty=0.0)
+            out[i] = res[-1]
+
+        th = [threading.Thread(target=run, args=(i,)) for i in range(2)]
+        [x.start() for x in th]
+        [x.join() for x in th]
+        for i in range(2):
+            st, body = out[i]
+            assert st["status_code"] == 200 and not st["has_error"], (st, body)
+            got = [int(x) for x in body["choices"][0]["message"]["content"].split()]
+            want = greedy(prompts[i])
+            assert len(got) >= n_new and got[:n_new] == want[:n_new], (got, want)
+    finally:
+        e.close()
+
+
+def test_trace_tool_with_a_pool_that_is_always_full(pkg, tmp_path):
+    """Up to four live requests of unequal lengths fed in portions of changing size beside single tokens of the others, in a pool that holds exactly what
+    the live requests need (each rounded up to 64 cells): a finished request's cells and state slot go to the next one at once.  Every position of every
+    request is asked for and compared with the restatement, in both precisions."""
+    cfg = S.config([S.retention(heads=4, dim=16, vdim=24, rot_dims=16, mlp=S.moe(experts=8, top=2, groups=(4, 2), ff=32)),
+                    S.attention(heads=6, kv_heads=3, dim=16, vdim=24, rel_rows=14, bias_max=100, mlp=S.moe(experts=4, top=1, groups=None, ff=48, shared=None)),
+                    S.attention_2(heads=4, kv_heads=2, dim=24, vdim=16, rot_dims=12, size=40, keep_first=6),
+                    S.retention(heads=2, dim=32, vdim=16, rot_dims=8)], width=88, vocab=211, loop=(1, 3, 2))
+    rig = Rig(pkg, tmp_path / "pool", cfg, seed=31)
+    V = cfg["vocab"]
+    rng = np.random.default_rng(5)
+    lengths = [150, 64, 97, 1, 33, 128, 70, 191, 2, 65]
+    reqs = {f"q{i}": toks(n, V, 300 + i) for i, n in enumerate(lengths)}
+    waiting, live, at = list(reqs), [], {}
+    steps, need = [], 0
+    while waiting or live:
+        while waiting and len(live) < 4:
+            r = waiting.pop(0)
+            live.append(r)
+            at[r] = 0
+        need = max(need, sum((len(reqs[r]) + 63) // 64 * 64 for r in live))
+        entries, end = [], []
+        for k, r in enumerate(live):
+            if len(live) > 1 and rng.random() < 0.2:
+                continue                                         # a request may sit a step out
+            n = int(rng.choice([1, 1, 1, 2, 3, 5, 17, 40])) if at[r] > 0 or k != 1 else len(reqs[r])
+            n = min(n, len(reqs[r]) - at[r])
+            entries.append({"id": r, "tokens": reqs[r][at[r]:at[r] + n], "want": list(range(n))})
+            at[r] += n
+            if at[r] == len(reqs[r]):
+                end.append(r)
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+        live = [r for r in live if r not in end]
+    want = {r: rig.ref(t) for r, t in reqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        out = tmp_path / dtype
+        p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", rig.dir, "--dtype", dtype, "--out", str(out), "--max-tokens", str(need)],
+                           input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600)
+        assert p.returncode == 0, p.stderr[-2000:]
+        got = {r: [] for r in reqs}
+        for st in steps:
+            if not any(e["want"] for e in st["entries"]):
+                continue
+            rows = np.fromfile(out / f"{st['step']}.f32", "<f4").reshape(-1, V)
+            k = 0
+            for e in st["entries"]:
+                got[e["id"]].append(rows[k:k + len(e["want"])])
+                k += len(e["want"])
+            assert k == len(rows)
+        errs = np.concatenate([row_errs(np.concatenate(got[r]), want[r]) for r in reqs])
+        if dtype == "float32":
+            assert errs.max() <= F32_WORST and np.percentile(errs, 90) <= F32_TOL, (errs.max(), np.percentile(errs, 90))
+        else:
+            assert np.median(errs) <= 2e-2 and np.percentile(errs, 90) <= BF16_TOL, (np.median(errs), np.percentile(errs, 90), errs.max())
