@@ -390,11 +390,54 @@ def tuterax_section(args) -> int:
     return 0
 
 
+def dinilorn_section(args) -> int:
+    """--dinilorn SIZES: prefill and decode throughput of synthetic Dinilorn models (bf16 weights, serving precision) beside the closest model this backend
+    already had - the Fidepel folder design of the same name: grouped-query attention on f32 cache rows, router-picked experts in groups plus a shared
+    expert, the same bf16 linear kernels, cell table and step function, equal width, depth, vocabulary, head and expert counts - with each side's distance
+    from its roofline: prefill as a fraction of the dense 16-bit matrix-core peak (2 FLOP per active weight and token), decode as a fraction of the HBM
+    peak (weight bytes one token reads).  One JSON line; the default workload of this script is untouched."""
+    import __graft_entry__ as ge
+    pkg = ge.load_pkg()
+    pkg.Backend()
+    ds, fs = pkg.dinilorn_synth, pkg.fidepel_synth
+    rows = []
+    for size in [x for x in args.dinilorn.split(",") if x]:
+        row = {"size": size, "prompt": args.prompt}
+        for name, mod, writer in (("dinilorn", ds, ds.write_synthetic_dinilorn), ("fidepel", fs, fs.write_synthetic_fidepel)):
+            s = mod.SIZES[size]
+            folder = os.path.join(args.model_dir, f"mi355-bench-{name}-{size}")
+            if not os.path.exists(os.path.join(folder, "model.safetensors")):
+                writer(folder, size, seed=0xC0FFEE)
+            cfg = mod.config_of(s)
+            wbytes = mod.weight_bytes_per_token(cfg)
+            flops_tok = wbytes - 2 * s.width                 # 2 FLOP per active weight = its bf16 bytes (the embedding row is a lookup)
+            kw = dict(n_ctx=args.ctx, n_batch=N_UBATCH, n_ubatch=N_UBATCH, n_seq_max=1)
+            m = pkg.Model(folder)
+            pf, dc, ms = _time_model(pkg, m, kw, args.prompt, args.steps, args.warmup, s.vocab)
+            m.close()
+            row["width"], row["layers"] = s.width, len(cfg["layers"])
+            row[name] = {"prefill_tok_s": round(pf, 1), "decode_tok_s": round(dc, 2), "ms_per_step": round(ms, 4), "weight_bytes_per_token": wbytes,
+                         "prefill_frac_of_mfma_peak": round(pf * flops_tok / (MFMA_BF16_PEAK_TFLOPS * 1e12), 4),
+                         "decode_frac_of_hbm_peak": round(wbytes * dc / (HBM_PEAK_GBPS * 1e9), 4)}
+            if not args.keep_model:
+                for f in (os.path.join(folder, "model.safetensors"), os.path.join(folder, "config.json")):
+                    if os.path.exists(f):
+                        os.remove(f)
+        a, b = row["dinilorn"], row["fidepel"]
+        row["roofline_ratio"] = {"prefill": round(a["prefill_frac_of_mfma_peak"] / max(b["prefill_frac_of_mfma_peak"], 1e-9), 3),
+                                 "decode": round(a["decode_frac_of_hbm_peak"] / max(b["decode_frac_of_hbm_peak"], 1e-9), 3)}
+        rows.append(row)
+    print(json.dumps({"metric": "dinilorn_prefill_decode_tok_s_vs_fidepel", "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                      "dtype": "bf16", "data": "synthetic", "higher_is_better": True, "sizes": rows}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--novorax", default="", help="comma list of synthetic Novorax sizes (w1024, w2048, w4096): time them beside an F16 Llama twin and exit")
     ap.add_argument("--fidepel", default="", help="comma list of synthetic Fidepel sizes (w1024, w2048, w4096): time them beside the Novorax model of that size and exit")
     ap.add_argument("--tuterax", default="", help="comma list of synthetic Tuterax sizes (w1024, w2048, w4096): time them beside the Novorax model of that size and exit")
+    ap.add_argument("--dinilorn", default="", help="comma list of synthetic Dinilorn sizes (w1024, w2048, w4096): time them beside the Fidepel model of that size and exit")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
@@ -440,6 +483,8 @@ def main() -> int:
         return fidepel_section(args)
     if args.tuterax:
         return tuterax_section(args)
+    if args.dinilorn:
+        return dinilorn_section(args)
 
     rank = int(os.environ.get("RANK", "0"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))
