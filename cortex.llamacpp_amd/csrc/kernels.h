@@ -299,6 +299,10 @@ hipError_t launch_moe_route_sigmoid_bias(const float *z, int ld_z, const float *
 // out[t][:] = sum_j w[t][j] * y[row(t, j)] [+ sigmoid(sg[t * ld_sg]) * b[t]]: the routed experts' weighted sum (rank order) and an always-on expert b (nullable)
 // behind its one-number gate; row(t, j) = slot_of[t * k + j], or t * k + j without a grouping
 hipError_t launch_moe_weighted_combine(float *out, const float *y, const float *w, const int32_t *slot_of, const float *b, const float *sg, int ld_sg, int T, int E, int k, hipStream_t st);
+// the same sum o[t][:] closed in one launch: x[t][:] += o / sqrt(mean(o^2) + eps) * (norm_off + norm_w) - the norm behind a feed-forward and the residual add
+constexpr int MOE_COMBINE_NORM_MAX_E = 12288, MOE_COMBINE_NORM_MAX_K = 64;   // widest row and most ranks the closing launch holds in LDS
+hipError_t launch_moe_weighted_combine_norm(float *x, const float *y, const float *w, const int32_t *slot_of, const float *b, const float *sg, int ld_sg,
+                                            const float *norm_w, float norm_off, float eps, int T, int E, int k, hipStream_t st);
 // x[t][:] += m * (a[t] + b[t] + sum_j w[t][j] * y[row(t, j)]): the close of a block whose mixer (a), always-on expert (b, nullable) and routed experts (y; k = 0:
 // none) all read the same normed input; row(t, j) = slot_of[t * k + j], or t * k + j without a grouping
 hipError_t launch_block_combine(float *x, const float *a, const float *b, const float *y, const float *w, const int32_t *slot_of, int T, int E, int k, float m, hipStream_t st);

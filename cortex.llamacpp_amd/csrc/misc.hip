@@ -686,6 +686,75 @@ hipError_t launch_moe_weighted_combine(float *out, const float *y, const float *
     return hipGetLastError();
 }
 
+// one workgroup of 1024 threads per token: the weighted sum into LDS with its sum of squares on the way, then the normed row joins the stream.  The k rows'
+// weights and places are read once into LDS; with VEC4 every thread owns four adjacent entries at a time and all its loads of a trip are independent of each
+// other (a single token's launch is one workgroup: what it costs is the number of dependent trips to memory)
+template <bool VEC4>
+__global__ __launch_bounds__(1024) void moe_weighted_combine_norm_kernel(float *x, const float *y, const float *w, const int32_t *slot_of, const float *b, const float *sg,
+                                                                         int ld_sg, const float *norm_w, float norm_off, float eps, int E, int k) {
+    extern __shared__ float row[];
+    __shared__ float part[16], sw[MOE_COMBINE_NORM_MAX_K];
+    __shared__ int srow[MOE_COMBINE_NORM_MAX_K];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    if (tid < k) { sw[tid] = w[(size_t)t * k + tid]; srow[tid] = slot_of ? slot_of[(size_t)t * k + tid] : t * k + tid; }
+    const float g = b ? (sg ? 1.0f / (1.0f + expf(-sg[(size_t)t * ld_sg])) : 1.0f) : 0.0f;
+    __syncthreads();
+    float ss = 0.0f;
+    if (VEC4) {
+        for (int d = 4 * tid; d < E; d += 4096) {
+            float4 o = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll 4
+            for (int j = 0; j < k; j++) {
+                const float4 v = *reinterpret_cast<const float4 *>(y + (size_t)srow[j] * E + d);
+                const float wj = sw[j];
+                o.x += v.x * wj; o.y += v.y * wj; o.z += v.z * wj; o.w += v.w * wj;
+            }
+            if (b) {
+                const float4 v = *reinterpret_cast<const float4 *>(b + (size_t)t * E + d);
+                o.x += g * v.x; o.y += g * v.y; o.z += g * v.z; o.w += g * v.w;
+            }
+            *reinterpret_cast<float4 *>(row + d) = o;
+            ss = fmaf(o.x, o.x, ss); ss = fmaf(o.y, o.y, ss); ss = fmaf(o.z, o.z, ss); ss = fmaf(o.w, o.w, ss);
+        }
+    } else {
+        for (int d = tid; d < E; d += 1024) {
+            float o = 0.0f;
+            for (int j = 0; j < k; j++) o += y[(size_t)srow[j] * E + d] * sw[j];
+            if (b) o += g * b[(size_t)t * E + d];
+            row[d] = o;
+            ss = fmaf(o, o, ss);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    if ((tid & 63) == 0) part[tid >> 6] = ss;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) tot += part[i];
+    const float inv = 1.0f / sqrtf(tot / (float)E + eps);
+    if (VEC4) {
+        for (int d = 4 * tid; d < E; d += 4096) {
+            const float4 o = *reinterpret_cast<const float4 *>(row + d), nw = *reinterpret_cast<const float4 *>(norm_w + d);
+            float4 xv = *reinterpret_cast<float4 *>(x + (size_t)t * E + d);
+            xv.x += o.x * inv * (norm_off + nw.x); xv.y += o.y * inv * (norm_off + nw.y); xv.z += o.z * inv * (norm_off + nw.z); xv.w += o.w * inv * (norm_off + nw.w);
+            *reinterpret_cast<float4 *>(x + (size_t)t * E + d) = xv;
+        }
+    } else {
+        for (int d = tid; d < E; d += 1024) x[(size_t)t * E + d] += row[d] * inv * (norm_off + norm_w[d]);
+    }
+}
+hipError_t launch_moe_weighted_combine_norm(float *x, const float *y, const float *w, const int32_t *slot_of, const float *b, const float *sg, int ld_sg,
+                                            const float *norm_w, float norm_off, float eps, int T, int E, int k, hipStream_t st) {
+    if ((int64_t)T * E <= 0) return hipSuccess;
+    if ((k > 0 && (!y || !w)) || !norm_w || E > MOE_COMBINE_NORM_MAX_E || k > MOE_COMBINE_NORM_MAX_K) return hipErrorInvalidValue;
+    const auto al16 = [](const void *p) { return !p || (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool vec4 = (E & 3) == 0 && al16(x) && al16(y) && al16(b) && al16(norm_w);
+    if (vec4) hipLaunchKernelGGL(moe_weighted_combine_norm_kernel<true>, dim3((unsigned)T), dim3(1024), (size_t)E * sizeof(float), st, x, y, w, slot_of, b, sg, ld_sg, norm_w, norm_off, eps, E, k);
+    else hipLaunchKernelGGL(moe_weighted_combine_norm_kernel<false>, dim3((unsigned)T), dim3(1024), (size_t)E * sizeof(float), st, x, y, w, slot_of, b, sg, ld_sg, norm_w, norm_off, eps, E, k);
+    return hipGetLastError();
+}
+
 // The close of a block whose sublayers all read one normed input: x[t][d] += m * (a[t][d] + b[t][d] + sum_j w[t][j] * y[row(t, j)][d]); a = the mixer's output,
 // b = an always-on expert's (nullable), y = the routed experts' rows (row(t, j) = slot_of[t * k + j], or t * k + j without a grouping; k = 0: none), added in
 // rank order.

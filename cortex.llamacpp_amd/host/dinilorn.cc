@@ -285,8 +285,10 @@ hipError_t Context::nvx_retention_mixer(const NvxLayer &L, const NvxRun &r, int 
     return hipSuccess;
 }
 
-// a routed feed-forward that reads its own norm: -> nvx_y_ = sum_j w_j expert_j(h) + sigmoid(gate) shared(h), h = norm2(x)
-hipError_t Context::nvx_routed_feed_forward(const NvxLayer &L, int T) {
+// a routed feed-forward that reads its own norm: sum_j w_j expert_j(h) + sigmoid(gate) shared(h), h = norm2(x); the sum, the norm behind it and the residual
+// add are one launch (x_ updated, *closed = true) where the row fits its LDS, else the sum lands in nvx_y_.  The shared expert touches no buffer of the routed
+// ones until the sum: in batches it runs on a side stream (fork behind the norm, join in front of the sum)
+hipError_t Context::nvx_routed_feed_forward(const NvxLayer &L, int T, bool *closed) {
     const NovoraxModel &M = *model->nvx;
     const int W = M.width;
     // up to MMB_VEC_ROWS rows every reader norms the stream itself (no launch for the norm); batches - and grouped expert batches, which gather normed rows -
@@ -297,12 +299,29 @@ hipError_t Context::nvx_routed_feed_forward(const NvxLayer &L, int T) {
         DNL_TRY(launch_rmsnorm_f32(x_, W, L.norm2, M.norm_off, nullptr, xn_, W, W, T, M.eps, stream_));
         h = xn_; pn = nullptr;
     }
-    const bool shared = L.shared_ff > 0;
+    // (steps of a few rows keep one stream: their launches are too short for the fork and the join to pay - measured)
+    const bool shared = L.shared_ff > 0, fork = nvx_fork_ok_ && shared && !profile_ && T > MMB_VEC_ROWS;
+    hipStream_t const main_stream = stream_;
+    struct Back { hipStream_t &s; hipStream_t v; ~Back() { s = v; } } back{stream_, main_stream};   // (every helper launches on stream_)
+    if (fork) {
+        DNL_TRY(hipEventRecord(nvx_fork_ev_, main_stream));
+        DNL_TRY(hipStreamWaitEvent(nvx_side_[0], nvx_fork_ev_, 0));
+        stream_ = nvx_side_[0];
+        DNL_TRY(nvx_shared_expert(L, h, pn, T));
+        DNL_TRY(hipEventRecord(nvx_join_ev_[0], nvx_side_[0]));
+        stream_ = main_stream;
+    }
     DNL_TRY(nvx_linear(L.route, h, W, T, nvx_a_, L.route.N, MMB_STORE, nullptr, 1.0f, pn));
     DNL_TRY(nvx_routed_experts(L, h, pn, T, nvx_a_, L.route.N));
-    if (shared) DNL_TRY(nvx_shared_expert(L, h, pn, T));
-    DNL_TRY(launch_moe_weighted_combine(nvx_y_, nvx_yg_, nvx_rw_, grouped ? nvx_slot_ : nullptr, shared ? nvx_ys_ : nullptr,
-                                        shared && L.off_sg >= 0 ? nvx_a_ + L.off_sg : nullptr, L.route.N, T, W, L.top, stream_));
+    if (fork) DNL_TRY(hipStreamWaitEvent(main_stream, nvx_join_ev_[0], 0));
+    else if (shared) DNL_TRY(nvx_shared_expert(L, h, pn, T));
+    const int32_t *slot_of = grouped ? nvx_slot_ : nullptr;
+    const float *sb = shared ? nvx_ys_ : nullptr, *sg = shared && L.off_sg >= 0 ? nvx_a_ + L.off_sg : nullptr;
+    if (closed && L.norm2b && W <= MOE_COMBINE_NORM_MAX_E && L.top <= MOE_COMBINE_NORM_MAX_K) {
+        DNL_TRY(launch_moe_weighted_combine_norm(x_, nvx_yg_, nvx_rw_, slot_of, sb, sg, L.route.N, L.norm2b, M.norm_off, M.eps, T, W, L.top, stream_));
+        *closed = true;
+    } else DNL_TRY(launch_moe_weighted_combine(nvx_y_, nvx_yg_, nvx_rw_, slot_of, sb, sg, L.route.N, T, W, L.top, stream_));
+    prof_mark("routed_feed_forward");
     return hipSuccess;
 }
 

@@ -346,7 +346,9 @@ bool Context::init_novorax(std::string &err) {
         nvx_ys_ = (float *)dalloc(T * W * 4);
         if (!nvx_sh_ || !nvx_ys_) { err = "shared expert buffers allocation failed"; return false; }
     }
-    if (M.parallel_block) {
+    bool side_branches = M.parallel_block;                      // (also: a routed feed-forward whose shared expert runs beside the routed ones)
+    for (const NvxLayer &L : M.layers) side_branches = side_branches || (L.ff_kind == NVX_FF_ROUTED && L.shared_ff > 0);
+    if (side_branches) {
         // side streams of the block's feed-forward branches (default priority, like the main one); MI355_BLOCK_FORK=0 keeps every launch on the main stream
         const char *ev = getenv("MI355_BLOCK_FORK");
         nvx_fork_ok_ = !(ev && ev[0] == '0');
@@ -467,10 +469,10 @@ hipError_t Context::nvx_linear(const BfMat &w, const float *x, int ldx, int T, f
     return launch_mmb(a, stream_);
 }
 
-hipError_t Context::nvx_feed_forward(const NvxLayer &L, int T) {
+hipError_t Context::nvx_feed_forward(const NvxLayer &L, int T, bool *closed) {
     const NovoraxModel &M = *model->nvx;
     const int W = M.width;
-    if (L.ff_kind == NVX_FF_ROUTED) return nvx_routed_feed_forward(L, T);
+    if (L.ff_kind == NVX_FF_ROUTED) return nvx_routed_feed_forward(L, T, closed);
     if (L.ff_kind == NVX_FF_DENSE) {
         if (L.gate.w) NVX_TRY(nvx_linear(L.gate, x_, W, T, nvx_ff_, L.ff, MMB_GELU_MUL, &L.up, 1.0f, L.norm2));
         else NVX_TRY(nvx_linear(L.up, x_, W, T, nvx_ff_, L.ff, MMB_RELU2, nullptr, 1.0f, L.norm2));
@@ -590,8 +592,9 @@ hipError_t Context::run_layers_novorax(int T) {
         // norm on the sublayer's output, added to the stream (norm1 / norm2 in front of a sublayer are nullptr in a design whose sublayers read the stream itself)
         NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm1b, 1.0f, x_, x_, W, W, T, eps, stream_));
         if (L.ff_kind != NVX_FF_NONE) {
-            NVX_TRY(nvx_feed_forward(L, T));
-            NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm2b, 1.0f, x_, x_, W, W, T, eps, stream_));
+            bool closed = false;
+            NVX_TRY(nvx_feed_forward(L, T, &closed));
+            if (!closed) NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm2b, 1.0f, x_, x_, W, W, T, eps, stream_));
             prof_mark("feed_forward");
         }
         if (debug_taps_ && dbg_) NVX_TRY(hipMemcpyAsync(dbg_ + (size_t)ir * cp.n_ubatch * W, x_, (size_t)T * W * 4, hipMemcpyDeviceToDevice, stream_));

@@ -183,8 +183,10 @@ class Context {
     hipError_t run_output_novorax(int n_out, int out_base);
     hipError_t nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi = MMB_STORE, const BfMat *w2 = nullptr, float out_scale = 1.0f,
                           const float *pn = nullptr, const float *bias = nullptr, float epi_limit = 0.0f);
-    hipError_t nvx_feed_forward(const NvxLayer &L, int T);
-    hipError_t nvx_routed_feed_forward(const NvxLayer &L, int T);            // dinilorn.cc: norm, [router ; shared gate] projection, routed + shared experts, weighted sum -> nvx_y_
+    // -> nvx_y_; *closed = true (closed given): the norm behind the feed-forward and the residual add were part of its last launch, x_ is already updated
+    hipError_t nvx_feed_forward(const NvxLayer &L, int T, bool *closed = nullptr);
+    // dinilorn.cc: norm, [router ; shared gate] projection, routed experts beside the shared expert (side stream), weighted sum + closing norm + residual add
+    hipError_t nvx_routed_feed_forward(const NvxLayer &L, int T, bool *closed);
     hipError_t nvx_retention_mixer(const NvxLayer &L, const NvxRun &r, int T);   // dinilorn.cc: projection, recurrence, gated unit-RMS output, W_o -> nvx_y_
     // fidepel.cc: a block whose mixer and feed-forward read one norm; grouped-query attention on the run's cache plane; experts picked by a router
     hipError_t nvx_parallel_block(const NvxLayer &L, const NvxRun &r, int T);
