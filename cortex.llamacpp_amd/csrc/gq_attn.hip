@@ -71,8 +71,8 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
         inv_k = 1.0f / sqrtf(gq_block_sum_256(ss, sh) / (float)NK + a.eps);
     }
     const float p = (float)a.tok_pos[t];
-    // (floor((p + 1) / every) as an integer division: exact)
-    const float q_temp = a.q_temp_every > 0 ? 1.0f + a.q_temp_coef * logf((float)((a.tok_pos[t] + 1) / a.q_temp_every) + 1.0f) : 1.0f;
+    // (positions are exact in f32 up to 2^24, and so is the floor of the correctly rounded quotient for a whole-number step)
+    const float q_temp = a.q_temp_every > 0.0f ? 1.0f + a.q_temp_coef * logf(floorf((p + 1.0f) / a.q_temp_every) + 1.0f) : 1.0f;
     if (tid < half) sincosf(p * a.rot_freq[tid], &cs[1][tid], &cs[0][tid]);
     const int vhalf = a.v_rot_freq ? a.vdim >> 1 : 0;
     if (tid >= 128 && tid - 128 < vhalf) {                       // (the upper waves: beside the key / query table of the lower ones)

@@ -320,7 +320,7 @@ struct GqPrepArgs {
     float q_scale; const float *head_scale;      // the query is multiplied by q_scale * head_scale[h] (nullable): the score's constant factors
     int maps;                              // score maps per head (0 or 1: one)
     int rot_neighbours;                    // 1: entry 2i turns with entry 2i + 1 instead of entry i with entry i + rot_dims / 2
-    float q_temp_coef; int q_temp_every;   // q_temp_every > 0: the query at position p is also multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)
+    float q_temp_coef, q_temp_every;       // q_temp_every > 0: the query at position p is also multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)
     const int32_t *tok_pos, *tok_cell;
     float *q; int ld_q;                    // [T][H*dim]: normed, turned, scaled queries
     float *cache;                          // [n_ctx][G*dim + G*vdim]

@@ -144,22 +144,22 @@ Model *dinilorn_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, s
                 if (!(L.softcap >= 0.0f)) { err = at + "mixer.softcap must not be negative"; return nullptr; }
                 const Json &qt = mx["q_temp"];
                 if (qt.is_object()) {
-                    L.q_temp_coef = (float)qt["coef"].as_double(0.0); L.q_temp_every = (int)qt["every"].as_int(0);
-                    if (L.q_temp_every < 1) { err = at + "q_temp.every must be positive"; return nullptr; }
+                    L.q_temp_coef = (float)qt["coef"].as_double(0.0); L.q_temp_every = (float)qt["every"].as_double(0.0);
+                    if (!(L.q_temp_every > 0.0f)) { err = at + "q_temp.every must be positive"; return nullptr; }
                 }
                 // distance d -> row of the bias table: one row per distance below B / 2, then rows spaced evenly in ln(d) up to bias_max (made in double; from
                 // bias_max on every distance takes the last row)
                 const int B = ld.rows_of(pm + "rel", H);
                 if (B < 0) break;
                 const int half = B / 2;
-                const int64_t far = mx["bias_max"].as_int(0);
-                if (B > 1 && !(far > half && far <= (1 << 24))) { err = at + "mixer.bias_max must lie above half the bias table's rows"; return nullptr; }
+                const double far = mx["bias_max"].as_double(0.0);
+                if (B > 1 && !(far > half && far <= (double)(1 << 24))) { err = at + "mixer.bias_max must lie above half the bias table's rows"; return nullptr; }
                 L.rel = ld.rows_f32({{pm + "rel", B}}, H);
                 L.rel_rows = B;
-                L.n_dist = B > 1 ? (int)far : 0;
+                L.n_dist = B > 1 ? (int)std::ceil(far) : 0;
                 std::vector<int32_t> bk((size_t)std::max(L.n_dist, 1), 0);
                 for (int n = 0; n < L.n_dist; n++)
-                    bk[(size_t)n] = n < half ? n : (int32_t)std::min<double>(B - 1, half + std::floor(std::log((double)n / half) / std::log((double)far / half) * (B - half)));
+                    bk[(size_t)n] = n < half ? n : (int32_t)std::min<double>(B - 1, half + std::floor(std::log((double)n / half) / std::log(far / half) * (B - half)));
                 L.dist_bucket = (int32_t *)ld.dev(bk.data(), bk.size() * 4);
                 std::vector<float> zero((size_t)H, 0.0f);           // one more term of score 0 in every head's softmax denominator
                 L.sink = (float *)ld.dev(zero.data(), zero.size() * 4);

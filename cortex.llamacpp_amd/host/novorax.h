@@ -101,7 +101,7 @@ struct NvxLayer {
     // longer distances take the last row); the first keep_first positions stay seen outside the window; rotary pairs (2i, 2i + 1); maps = 2: two score maps
     // per head ([head][map][dim] rows of q and k) joined as unit_rms(a1 - map_lambda a2) * map_mult; the gate holds one number per output entry
     float *proj_bias = nullptr, *o_bias = nullptr;
-    float q_temp_coef = 0.0f; int q_temp_every = 0;
+    float q_temp_coef = 0.0f, q_temp_every = 0.0f;
     float *rel = nullptr; int32_t *dist_bucket = nullptr; int n_dist = 0, rel_rows = 0;
     int keep_first = 0, maps = 1;
     bool rot_neighbours = false, gate_per_entry = false;
