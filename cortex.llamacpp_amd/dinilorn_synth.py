@@ -51,7 +51,7 @@ def config_of(s: DinilornSize) -> dict:
     layers = []
     for code in s.pattern:
         if code[0] == "R":
-            lc = {"type": "retention", "mixer": {"decay": [float(1.0 - 2.0 ** (-5 - 3 * h / max(s.r_heads - 1, 1))) for h in range(s.r_heads)], "dim": s.r_dim, "heads": s.r_heads,
+            lc = {"type": "retention", "mixer": {"decay": [float(1.0 - 0.75 * 2.0 ** (-5 - 3 * h / max(s.r_heads - 1, 1))) for h in range(s.r_heads)], "dim": s.r_dim, "heads": s.r_heads,
                                                  "rot": {"base": 500000.0, "dims": s.r_dim}, "vdim": s.r_vdim}}
         elif code[0] == "A":
             lc = {"type": "attention", "mixer": {"bias_max": s.bias_max, "dim": s.dim, "heads": s.heads, "kv_heads": s.kv_heads, "q_temp": {"coef": 0.1, "every": 256},

@@ -21,7 +21,7 @@ def moe(experts=6, top=2, groups=(3, 2), ff=24, limit=1.2, shared=(40, 1.6)):
 
 
 def retention(heads=3, dim=20, vdim=12, rot_dims=8, base=5000.0, decay=None, mlp=None):
-    mixer = {"decay": list(decay) if decay else [1.0 - 2.0 ** (-3 - h) for h in range(heads)], "dim": dim, "heads": heads, "vdim": vdim}
+    mixer = {"decay": list(decay) if decay else [1.0 - 0.3 * 2.0 ** (-1 - h) for h in range(heads)], "dim": dim, "heads": heads, "vdim": vdim}
     if rot_dims:
         mixer["rot"] = {"base": base, "dims": rot_dims}
     return {"type": "retention", "mixer": mixer, "mlp": mlp}

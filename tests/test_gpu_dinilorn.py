@@ -152,13 +152,13 @@ def test_the_restatement_tells_the_parts_apart(pkg, tmp_path):
 
 
 def test_the_router_alone(pkg, tmp_path):
-    """Twelve experts in four groups with selection biases from -3 to 2: choice scores that are negative, best experts inside closed groups, groups that win
+    """Fifteen experts in five groups with selection biases from -3 to 2: choice scores that are negative, best experts inside closed groups, groups that win
     by their second best.  The stream behind the feed-forward and the logits agree with the restatement; the restatement without the bias, or with every
     group open, does not."""
-    E, top = 12, 3
-    mlp = S.moe(experts=E, top=top, groups=(4, 2), ff=8, shared=None)
+    E, top = 15, 4
+    mlp = S.moe(experts=E, top=top, groups=(5, 2), ff=8, shared=None)
     rig = Rig(pkg, tmp_path / "router", S.config([S.retention(heads=1, dim=8, vdim=8, rot_dims=0, mlp=mlp)], width=48, vocab=200), seed=21,
-              tweak=lambda W: W.__setitem__("l0.mlp.correction", torch.tensor([-3.0, 0.4, -0.2, 0.9, 0.0, -1.5, 0.3, 0.3, 2.0, -2.0, -2.0, 0.1]).to(torch.bfloat16)))
+              tweak=lambda W: W.__setitem__("l0.mlp.correction", torch.tensor([-3.0, 0.4, -0.2, 0.9, 0.0, -1.5, 0.3, 0.3, 2.0, -2.0, -2.0, 0.1, 0.6, -0.4, 1.1]).to(torch.bfloat16)))
     t = toks(120, 200, 3)
     want, taps = rig.ref(t, layers=True)
     c = rig.ctx(n_ubatch=128)
@@ -431,7 +431,7 @@ def test_a_windowed_request_beside_requests_that_come_and_go(pkg, tmp_path):
 def test_a_memory_that_holds_hundreds_of_tokens(pkg, tmp_path):
     """Decays close to one: what token 60 wrote is still read 240 and more tokens later (the restatement with another token there differs at those rows) -
     through micro-batches, portions of two and single tokens."""
-    cfg = S.config([S.retention(heads=2, dim=24, vdim=16, rot_dims=8, decay=[0.9990234375, 0.99951171875])], width=48, vocab=50)
+    cfg = S.config([S.retention(heads=2, dim=24, vdim=16, rot_dims=8, decay=[0.99853515625, 0.99951171875])], width=48, vocab=50)
     rig = Rig(pkg, tmp_path / "hold", cfg, seed=5)
     t = toks(330, 50, 17)
     want = rig.ref(t)
@@ -629,10 +629,16 @@ def test_trace_tool_with_a_pool_that_is_always_full(pkg, tmp_path):
     the live requests need (each rounded up to 64 cells): a finished request's cells and state slot go to the next one at once.  Every position of every
     request is asked for and compared with the restatement, in both precisions."""
     cfg = S.config([S.retention(heads=4, dim=16, vdim=24, rot_dims=16, mlp=S.moe(experts=8, top=2, groups=(4, 2), ff=32)),
-                    S.attention(heads=6, kv_heads=3, dim=16, vdim=24, rel_rows=14, bias_max=100, mlp=S.moe(experts=4, top=1, groups=None, ff=48, shared=None)),
+                    S.attention(heads=6, kv_heads=3, dim=16, vdim=24, rel_rows=14, bias_max=100, mlp=S.moe(experts=4, top=2, groups=None, ff=48)),
                     S.attention_2(heads=4, kv_heads=2, dim=24, vdim=16, rot_dims=12, size=40, keep_first=6),
                     S.retention(heads=2, dim=32, vdim=16, rot_dims=8)], width=88, vocab=211, loop=(1, 3, 2))
-    rig = Rig(pkg, tmp_path / "pool", cfg, seed=31)
+    def tweak(W):
+        # selection biases spread wide: few tokens sit within a bf16 rounding of a routing edge, so the serving precision is measured on its arithmetic and
+        # not on how many experts flipped (a flip moves a row - and through the retention state every later row - by far more than rounding does)
+        for name in [n for n in W if n.endswith("mlp.correction")]:
+            E = W[name].numel()
+            W[name] = torch.linspace(-1.5, 1.5, E)[torch.randperm(E, generator=torch.Generator().manual_seed(E))].to(torch.bfloat16)
+    rig = Rig(pkg, tmp_path / "pool", cfg, seed=31, tweak=tweak)
     V = cfg["vocab"]
     rng = np.random.default_rng(5)
     lengths = [150, 64, 97, 1, 33, 128, 70, 191, 2, 65]
