@@ -17,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 EXPERIMENTS = os.environ.get("MI355_BUILD_EXPERIMENTS", "0") == "1"
 SRC = [
     "csrc/mmvq.hip", "csrc/mmvq_fast.hip", "csrc/mmvq_stream.hip", "csrc/mmq.hip", "csrc/mmq_q80.hip", "csrc/act.hip", "csrc/misc.hip", "csrc/mmf.hip", "csrc/attn.hip", "csrc/attn_out.hip", "csrc/attn_prefill.hip", "csrc/clip.hip",
-    "csrc/mmb.hip", "csrc/latent_attn.hip", "csrc/mlstm.hip", "csrc/gq_attn.hip", "csrc/delta_rule.hip", "csrc/retention.hip",
+    "csrc/mmb.hip", "csrc/latent_attn.hip", "csrc/mlstm.hip", "csrc/gq_attn.hip", "csrc/delta_rule.hip", "csrc/retention.hip", "csrc/routed_ff.hip",
 ] + (["csrc/decode_engine.hip", "csrc/decode_mega.hip"] if EXPERIMENTS else ["csrc/experiments_absent.cc"]) + [
     "host/gguf.cc", "host/runtime.cc", "host/novorax.cc", "host/fidepel.cc", "host/tuterax.cc", "host/dinilorn.cc", "host/tp_comm.cc", "host/vocab.cc", "host/sampling.cc", "host/grammar.cc", "host/json_schema.cc", "host/log.cc", "host/server_context.cc", "host/engine.cc",
     "host/hip_backend.cc", "host/tp_split.cc", "host/clip.cc", "host/image_decode.cc", "csrc/c_api.cc",
@@ -43,7 +43,7 @@ EXTRA = {
 }
 # float code of these files is kept off the packed-f32 instructions (v_pk_fma_f32 and its kin): their whole arithmetic is f32 and must be the scalar forms
 NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-for _s in ("csrc/mmb.hip", "csrc/latent_attn.hip", "csrc/mlstm.hip", "csrc/gq_attn.hip", "csrc/delta_rule.hip", "csrc/retention.hip"):
+for _s in ("csrc/mmb.hip", "csrc/latent_attn.hip", "csrc/mlstm.hip", "csrc/gq_attn.hip", "csrc/delta_rule.hip", "csrc/retention.hip", "csrc/routed_ff.hip"):
     EXTRA[_s] = EXTRA.get(_s, []) + NO_PACKED_F32
 
 

@@ -292,7 +292,7 @@ hipError_t launch_moe_uniform_combine(float *out, const float *y, const int32_t 
 // largest s, only experts of the `keep` best groups can be taken; the k best of them, weights s / (their sum + 1e-20) * scale.  ids / w: [T][k], best first.
 constexpr int MOE_ROUTE_MAX_EXPERTS = 8192;
 hipError_t launch_moe_route_groups(const float *z, int ld_z, int T, int E, int k, int n_group, int keep, float scale, int32_t *ids, float *w, hipStream_t st);
-// router with a selection bias (misc.hip): s = sigmoid(z[t][0 .. E)); the choice score of an expert is c = s + bias (bias nullable; c may be negative); the experts
+// router with a selection bias (routed_ff.hip, like the two launches behind it): s = sigmoid(z[t][0 .. E)); the choice score of an expert is c = s + bias (bias nullable; c may be negative); the experts
 // form n_group equal groups of neighbours, a group scores as the sum of its two largest c (its only one if it holds one expert), only experts of the `keep`
 // best groups can be taken; the k open experts with the largest c, lowest index first on a tie; weights = their s as it is.  ids / w: [T][k], best first.
 hipError_t launch_moe_route_sigmoid_bias(const float *z, int ld_z, const float *bias, int T, int E, int k, int n_group, int keep, int32_t *ids, float *w, hipStream_t st);
@@ -339,7 +339,7 @@ struct GqAttnArgs {
     int window;                            // cells at distance 0 .. window - 1 are seen; 0 = every earlier cell
     int keep_first;                        // with a window: cells at positions below keep_first stay seen at any distance
     int maps;                              // score maps per head (0 or 1: one); H counts (head, map) pairs, G the value heads
-    // nullable: a learned bias per (distance bucket, head) added to the score behind the soft cap: rel[bucket(d) * rel_heads + h], bucket(d) = dist_bucket[d]
+    // nullable: a learned bias per (distance bucket, head) added to the score behind the soft cap: rel[bucket(d) * H + h], bucket(d) = dist_bucket[d]
     // for d < n_dist, else rel_rows - 1
     const float *rel; const int32_t *dist_bucket; int n_dist, rel_rows;
     const float *sink;                     // [H] or nullptr: a logit without key or value in the softmax denominator
