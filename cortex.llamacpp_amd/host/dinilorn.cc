@@ -321,7 +321,7 @@ hipError_t Context::nvx_routed_feed_forward(const NvxLayer &L, int T, bool *clos
         DNL_TRY(launch_moe_weighted_combine_norm(x_, nvx_yg_, nvx_rw_, slot_of, sb, sg, L.route.N, L.norm2b, M.norm_off, M.eps, T, W, L.top, stream_));
         *closed = true;
     } else DNL_TRY(launch_moe_weighted_combine(nvx_y_, nvx_yg_, nvx_rw_, slot_of, sb, sg, L.route.N, T, W, L.top, stream_));
-    prof_mark("routed_feed_forward");
+    prof_mark("expert_sum_norm");
     return hipSuccess;
 }
 
