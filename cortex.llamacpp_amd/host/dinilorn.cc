@@ -139,7 +139,7 @@ Model *dinilorn_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, s
             const int NQ = H * L.maps * D, NK = G * L.maps * D, NV = G * VD;
             L.off_gate = NQ + NK + NV;
             if (L.maps == 1) {
-                if (L.rot_dims > 0) { err = at + "this attention takes no rotation"; return nullptr; }
+                L.rot_dims = 0; L.rot_freq = nullptr;           // (positions enter this attention through the multiplier and the bias only)
                 L.softcap = (float)mx["softcap"].as_double(0.0);
                 if (!(L.softcap >= 0.0f)) { err = at + "mixer.softcap must not be negative"; return nullptr; }
                 const Json &qt = mx["q_temp"];
